@@ -32,6 +32,8 @@ def register_model(name: str, config_class, build, model_type: str = None) -> No
 
 def architecture_of(config_dict: Dict[str, Any]) -> Architecture:
     archs = config_dict.get("architectures")
+    if not archs and isinstance(config_dict.get("architecture"), str):
+        archs = [config_dict["architecture"]]           # (a config.json that names one, as a string)
     if not archs and config_dict.get("model_type") in MODEL_TYPE_ALIASES:
         archs = [MODEL_TYPE_ALIASES[config_dict["model_type"]]]
     if not archs:

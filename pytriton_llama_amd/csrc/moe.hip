@@ -1,0 +1,474 @@
+// A routed feed-forward (mixture of experts) that never leaves the device, so that a step with
+// one can be recorded as a graph:
+//
+//   ptl_moe_topk      per token: scores = sigmoid(logits) in float32, the ``top`` largest, their
+//                     experts and scores (the score is the weight, with or without a
+//                     renormalisation over the chosen ones); and the sigmoid of extra logit columns
+//                     behind the experts' (a gate of a shared expert)
+//   ptl_moe_sort      the (token, choice) pairs ordered by expert: positions, the tiles of
+//                     MOE_TM rows that the products walk, all by one workgroup
+//   ptl_moe_gate_up   per tile: rows gathered from x, the expert's gate and up matrices, and
+//                     the gated activation, written in sorted order. The routing weight scales
+//                     the expert's input (it is applied to both products, which are linear) or
+//                     is left for the output
+//   ptl_moe_down      per tile: the expert's down matrix on the sorted rows
+//   ptl_moe_combine   per token: the sum of its choices' rows (times the weight when it scales
+//                     the output), plus gate * a shared expert's row
+//   ptl_gated_act     the experts' activation on a dense [T, 2I] gate|up product
+//
+// Activation kinds: 0: silu(g) * u;  1: g' = min(g, limit), u' = clamp(u, -limit, limit),
+// g' * sigmoid(1.702 g') * (u' + 1).
+#include "common.h"
+#include "mfma.h"
+#include <math.h>
+
+#define MOE_TM 64
+#define MOE_SORT_LDS 8192      // pairs whose experts the sorting workgroup holds in LDS
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+__device__ __forceinline__ float gated_act(int kind, float g, float u, float limit) {
+  if (kind == 1) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * sigmoidf_(1.702f * g) * (u + 1.0f);
+  }
+  return g * sigmoidf_(g) * u;
+}
+
+// One wave a token. Lane l holds the logits of experts l, l + 64, ...
+#define TOPK_PER_LANE 16
+__global__ void __launch_bounds__(256)
+moe_topk_kernel(const float* __restrict__ logits, int ld, int T_, int E, int top, int extra,
+                int renormalize, int32_t* __restrict__ idx, float* __restrict__ wgt,
+                float* __restrict__ extra_out) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (t >= T_) return;
+  const float* z = logits + (size_t)t * ld;
+  float v[TOPK_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < TOPK_PER_LANE; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < E ? z[e] : -INFINITY;
+  }
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E && (v[i] > best || (v[i] == best && e < at)) && v[i] != -INFINITY) {
+        best = v[i];
+        at = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oa = __shfl_xor(at, o, 64);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    if (at >= E) at = k;                 // (only when a logit is NaN: the NaN then shows in the output)
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i)
+      if (lane + 64 * i == at) v[i] = -INFINITY;
+    const float s = sigmoidf_(best);
+    sum += s;
+    if (lane == 0) {
+      idx[(size_t)t * top + k] = at;
+      wgt[(size_t)t * top + k] = s;
+    }
+  }
+  if (renormalize && lane == 0)
+    for (int k = 0; k < top; ++k) wgt[(size_t)t * top + k] /= sum;
+  if (lane < extra) extra_out[(size_t)t * extra + lane] = sigmoidf_(z[E + lane]);
+}
+
+extern "C" int ptl_moe_topk(const float* logits, int ld, int T_, int E, int top, int extra, int renormalize,
+                            int32_t* idx, float* wgt, float* extra_out, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (E <= 0 || top <= 0 || top > E || E > 64 * TOPK_PER_LANE || extra < 0 || extra > 64 || ld < E + extra ||
+      (extra && !extra_out))
+    return PTL_ERR_ARG;
+  moe_topk_kernel<<<(T_ + 3) / 4, 256, 0, st>>>(logits, ld, T_, E, top, extra, renormalize, idx, wgt, extra_out);
+  return ptl_launch_status();
+}
+
+// One workgroup. A = pairs (token, choice). Writes: pos_of[a] (the sorted position of pair a),
+// sorted[p] (the pair at position p), expert_end[e] (one past the last position of expert e),
+// and the tile list: tile_expert[i] (-1: no tile), tile_row0[i] for i < max_tiles.
+__global__ void __launch_bounds__(1024)
+moe_sort_kernel(const int32_t* __restrict__ idx, int A, int E, int32_t* __restrict__ pos_of,
+                int32_t* __restrict__ sorted, int32_t* __restrict__ expert_end,
+                int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0, int max_tiles) {
+  extern __shared__ int32_t sh[];        // count [E], start [E], n_tiles [1], experts of the pairs [A]
+  int32_t* count = sh;
+  int32_t* start = sh + E;
+  int32_t* n_tiles = sh + 2 * E;
+  int32_t* lidx = sh + 2 * E + 1;
+  for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
+  __syncthreads();
+  for (int a = threadIdx.x; a < A; a += 1024) {
+    const int e = idx[a];
+    if (e >= 0 && e < E) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tile = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = count[e];
+      start[e] = at;
+      for (int r = 0; r < c && tile < max_tiles; r += MOE_TM, ++tile) {
+        tile_expert[tile] = e;
+        tile_row0[tile] = at + r;
+      }
+      at += c;
+      expert_end[e] = at;
+      count[e] = 0;                      // from here on: the places of the expert handed out
+    }
+    *n_tiles = tile;
+  }
+  __syncthreads();
+  for (int i = *n_tiles + threadIdx.x; i < max_tiles; i += 1024) {
+    tile_expert[i] = -1;
+    tile_row0[i] = 0;
+  }
+  // places inside an expert in the order of the pairs, so that the layout does not change from
+  // run to run: with the experts of all pairs in LDS, thread e walks them and hands expert e's
+  // places out in order (every thread reads the same word: a broadcast). More pairs than LDS
+  // holds: places by atomic counters (the order inside an expert then varies, the results
+  // of a row do not depend on its place).
+  if (A <= MOE_SORT_LDS) {
+    for (int a = threadIdx.x; a < A; a += 1024) lidx[a] = idx[a];
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += 1024) {
+      int p = start[e];
+      const int end = expert_end[e];
+      for (int a = 0; a < A && p < end; ++a)
+        if (lidx[a] == e) {
+          sorted[p] = a;
+          pos_of[a] = p++;
+        }
+    }
+    return;
+  }
+  for (int a = threadIdx.x; a < A; a += 1024) {
+    const int e = idx[a];
+    if (e < 0 || e >= E) continue;
+    const int p = start[e] + atomicAdd(&count[e], 1);
+    sorted[p] = a;
+    pos_of[a] = p;
+  }
+}
+
+extern "C" int ptl_moe_max_tiles(int A, int E) { return (A + MOE_TM - 1) / MOE_TM + (A < E ? A : E); }
+
+extern "C" int ptl_moe_sort(const int32_t* idx, int A, int E, int32_t* pos_of, int32_t* sorted,
+                            int32_t* expert_end, int32_t* tile_expert, int32_t* tile_row0, int max_tiles,
+                            hipStream_t st) {
+  if (A <= 0) return PTL_OK;
+  if (E <= 0 || E > 8192 || max_tiles < ptl_moe_max_tiles(A, E)) return PTL_ERR_ARG;
+  moe_sort_kernel<<<1, 1024, (2 * E + 1 + (A <= MOE_SORT_LDS ? A : 0)) * sizeof(int32_t), st>>>(idx, A, E, pos_of, sorted, expert_end,
+                                                                  tile_expert, tile_row0, max_tiles);
+  return ptl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// The experts' products over the tile list. Vector-FMA form (any sizes, both dtypes): a tile of
+// MOE_TM sorted rows x 64 result columns a workgroup; the gate|up product keeps two sums an
+// output (gate row n and up row I + n of the expert's [2 I, K] matrix).
+#define MK 16
+
+template <typename T, bool GATE_UP>
+__global__ void __launch_bounds__(256)
+moe_gemm_kernel(T* __restrict__ out, long ldo, const T* __restrict__ x, long ldx, const T* __restrict__ w,
+                const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
+                const int32_t* __restrict__ expert_end, const int32_t* __restrict__ sorted,
+                const float* __restrict__ wgt, int top, int N, int K, int act, float limit) {
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  const int row0 = tile_row0[blockIdx.y];
+  const int rows = min(MOE_TM, expert_end[e] - row0);
+  __shared__ float As[MK][MOE_TM + 4];
+  __shared__ float Bs[GATE_UP ? 2 : 1][MK][64 + 4];
+  __shared__ int32_t src_row[MOE_TM];
+  __shared__ float row_w[MOE_TM];
+  const int tid = threadIdx.x;
+  if (tid < MOE_TM) {
+    int r = -1;
+    float f = 1.f;
+    if (tid < rows) {
+      if (GATE_UP) {
+        const int a = sorted[row0 + tid];
+        r = a / top;
+        if (wgt) f = wgt[a];
+      } else {
+        r = row0 + tid;
+      }
+    }
+    src_row[tid] = r;
+    row_w[tid] = f;
+  }
+  __syncthreads();
+  const int n0 = blockIdx.x * 64;
+  const size_t wrows = GATE_UP ? 2 * (size_t)N : (size_t)N;
+  w += (size_t)e * wrows * K;
+  const int lr = tid >> 2, lk = (tid & 3) << 2;
+  const int ty = tid >> 4, tx = tid & 15;
+  float acc[GATE_UP ? 2 : 1][4][4];
+#pragma unroll
+  for (int g = 0; g < (GATE_UP ? 2 : 1); ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[g][i][j] = 0.f;
+  const int my_src = src_row[lr];
+  for (int k0 = 0; k0 < K; k0 += MK) {
+    const int n = n0 + lr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + lk + i;
+      As[lk + i][lr] = (my_src >= 0 && k < K) ? to_float<T>(x[(size_t)my_src * ldx + k]) : 0.f;
+      Bs[0][lk + i][lr] = (n < N && k < K) ? to_float<T>(w[(size_t)n * K + k]) : 0.f;
+      if (GATE_UP) Bs[1][lk + i][lr] = (n < N && k < K) ? to_float<T>(w[((size_t)N + n) * K + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < MK; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int g = 0; g < (GATE_UP ? 2 : 1); ++g) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = Bs[g][k][tx * 4 + j];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[g][i][j] = fmaf(a[i], b[j], acc[g][i][j]);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = ty * 4 + i;
+    if (m >= rows) continue;
+    const float f = row_w[m];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= N) continue;
+      float v;
+      if (GATE_UP)
+        v = gated_act(act, acc[0][i][j] * f, acc[GATE_UP ? 1 : 0][i][j] * f, limit);
+      else
+        v = acc[0][i][j];
+      out[(size_t)(row0 + m) * ldo + n] = from_float<T>(v);
+    }
+  }
+}
+
+// Matrix-core form for bfloat16 (K % 8 == 0, aligned rows): a wave owns 16 sorted rows x 64
+// columns, fragments straight from memory as in ptl_gemm_heads_nt.
+template <bool GATE_UP>
+__global__ void __launch_bounds__(256)
+moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restrict__ x, long ldx,
+                     const bf16_t* __restrict__ w, const int32_t* __restrict__ tile_expert,
+                     const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ expert_end,
+                     const int32_t* __restrict__ sorted, const float* __restrict__ wgt, int top, int N, int K,
+                     int act, float limit) {
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int ln = lane & 15, lg = lane >> 4;
+  const int row0 = tile_row0[blockIdx.y] + 16 * wave;
+  const int rows = min(16, expert_end[e] - row0);
+  if (rows <= 0) return;
+  const int n0 = blockIdx.x * 64;
+  const size_t wrows = GATE_UP ? 2 * (size_t)N : (size_t)N;
+  w += (size_t)e * wrows * K;
+  const int mr = min(ln, rows - 1);
+  int src = row0 + mr;
+  float f = 1.f;
+  if (GATE_UP) {
+    const int a = sorted[src];
+    src = a / top;
+    if (wgt) f = wgt[a];
+  }
+  const bf16_t* arow = x + (size_t)src * ldx;
+  const bf16_t* brow[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) brow[j] = w + (size_t)min(n0 + 16 * j + ln, N - 1) * K;
+  f32x4_t acc[GATE_UP ? 2 : 1][4];
+#pragma unroll
+  for (int g = 0; g < (GATE_UP ? 2 : 1); ++g)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[g][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const size_t up = (size_t)N * K;
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int k = k0 + 8 * lg;
+    Frag8 a, b[GATE_UP ? 2 : 1][4];
+    a.u = k < K ? *reinterpret_cast<const uint4*>(arow + k) : zero;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      b[0][j].u = k < K ? load_once(brow[j] + k) : zero;
+      if (GATE_UP) b[GATE_UP ? 1 : 0][j].u = k < K ? load_once(brow[j] + up + k) : zero;
+    }
+#pragma unroll
+    for (int g = 0; g < (GATE_UP ? 2 : 1); ++g)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[g][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[g][j].v, a.v, acc[g][j], 0, 0, 0);
+  }
+  if (ln < rows) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 16 * j + 4 * lg + i;
+        if (n >= N) continue;
+        float v;
+        if (GATE_UP)
+          v = gated_act(act, acc[0][j][i] * f, acc[GATE_UP ? 1 : 0][j][i] * f, limit);
+        else
+          v = acc[0][j][i];
+        out[(size_t)(row0 + ln) * ldo + n] = float_to_bf16(v);
+      }
+  }
+}
+
+static bool mfma_ok(const void* x, long ldx, const void* w, int K) {
+  return K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x | (uintptr_t)w) % 16 == 0;
+}
+
+// out [A, I] (sorted order) = act(w_a * x[token] Wg_e^T, w_a * x[token] Wu_e^T); w [E, 2 I, K];
+// wgt null: the routing weight is not applied here.
+extern "C" int ptl_moe_gate_up(void* out, long ldo, const void* x, long ldx, const void* w,
+                               const int32_t* tile_expert, const int32_t* tile_row0,
+                               const int32_t* expert_end, const int32_t* sorted, const float* wgt,
+                               int max_tiles, int top, int I, int K, int act, float limit, int dtype,
+                               hipStream_t st) {
+  if (max_tiles <= 0) return PTL_OK;
+  if (I <= 0 || K <= 0 || top <= 0 || max_tiles > 65535) return PTL_ERR_ARG;
+  dim3 grid((I + 63) / 64, max_tiles);
+  if (dtype == PTL_DTYPE_F32)
+    moe_gemm_kernel<float, true><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
+                                                       tile_expert, tile_row0, expert_end, sorted, wgt, top, I,
+                                                       K, act, limit);
+  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
+    moe_gemm_mfma_kernel<true><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                     (const bf16_t*)w, tile_expert, tile_row0, expert_end,
+                                                     sorted, wgt, top, I, K, act, limit);
+  else if (dtype == PTL_DTYPE_BF16)
+    moe_gemm_kernel<bf16_t, true><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                        (const bf16_t*)w, tile_expert, tile_row0, expert_end,
+                                                        sorted, wgt, top, I, K, act, limit);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}
+
+// out [A, N] (sorted order) = x [A, K] (sorted order) Wd_e^T; w [E, N, K]
+extern "C" int ptl_moe_down(void* out, long ldo, const void* x, long ldx, const void* w,
+                            const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* expert_end,
+                            int max_tiles, int N, int K, int dtype, hipStream_t st) {
+  if (max_tiles <= 0) return PTL_OK;
+  if (N <= 0 || K <= 0 || max_tiles > 65535) return PTL_ERR_ARG;
+  dim3 grid((N + 63) / 64, max_tiles);
+  if (dtype == PTL_DTYPE_F32)
+    moe_gemm_kernel<float, false><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
+                                                        tile_expert, tile_row0, expert_end, nullptr, nullptr, 1,
+                                                        N, K, 0, 0.f);
+  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
+    moe_gemm_mfma_kernel<false><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                      (const bf16_t*)w, tile_expert, tile_row0, expert_end,
+                                                      nullptr, nullptr, 1, N, K, 0, 0.f);
+  else if (dtype == PTL_DTYPE_BF16)
+    moe_gemm_kernel<bf16_t, false><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                         (const bf16_t*)w, tile_expert, tile_row0, expert_end,
+                                                         nullptr, nullptr, 1, N, K, 0, 0.f);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}
+
+// y[t, :] = sum_k f_k * rows[pos_of[t * top + k], :] + gate[t * ldg] * shared[t, :], float32.
+// f_k = wgt[t * top + k] when wgt is given (the weight scales the expert's output), else 1.
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_combine_kernel(float* __restrict__ y, const T* __restrict__ rows, long ldr, const int32_t* __restrict__ pos_of,
+                   const float* __restrict__ wgt, int top, const T* __restrict__ shared,
+                   const float* __restrict__ gate, int ldg, int N) {
+  const size_t t = blockIdx.y;
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  float s = 0.f;
+  for (int k = 0; k < top; ++k) {
+    const float v = to_float<T>(rows[(size_t)pos_of[t * top + k] * ldr + n]);
+    s += wgt ? v * wgt[t * top + k] : v;
+  }
+  if (shared) {
+    const float v = to_float<T>(shared[t * N + n]);
+    s += gate ? v * gate[t * ldg] : v;
+  }
+  y[t * N + n] = s;
+}
+
+extern "C" int ptl_moe_combine(float* y, const void* rows, long ldr, const int32_t* pos_of, const float* wgt,
+                               int top, const void* shared, const float* gate, int ldg, int T_, int N, int dtype,
+                               hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (N <= 0 || top <= 0 || T_ > 65535 * 64) return PTL_ERR_ARG;
+  for (int t0 = 0; t0 < T_; t0 += 65535) {
+    const int nt = T_ - t0 < 65535 ? T_ - t0 : 65535;
+    dim3 grid((N + 255) / 256, nt);
+    const size_t o = (size_t)t0;
+    if (dtype == PTL_DTYPE_F32)
+      moe_combine_kernel<float><<<grid, 256, 0, st>>>(
+          y + o * N, (const float*)rows, ldr, pos_of + o * top, wgt ? wgt + o * top : nullptr, top,
+          shared ? (const float*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg, N);
+    else if (dtype == PTL_DTYPE_BF16)
+      moe_combine_kernel<bf16_t><<<grid, 256, 0, st>>>(
+          y + o * N, (const bf16_t*)rows, ldr, pos_of + o * top, wgt ? wgt + o * top : nullptr, top,
+          shared ? (const bf16_t*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg, N);
+    else
+      return PTL_ERR_ARG;
+  }
+  return ptl_launch_status();
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_act_kernel(T* __restrict__ out, const T* __restrict__ gu, int I, size_t total, int act, float limit) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * 256;
+  for (; i < total; i += step) {
+    const size_t t = i / I;
+    const int c = (int)(i - t * I);
+    out[i] = from_float<T>(gated_act(act, to_float<T>(gu[t * 2 * I + c]), to_float<T>(gu[t * 2 * I + I + c]), limit));
+  }
+}
+
+// out [T, I] = act(gu[:, :I], gu[:, I:]) for a dense gate|up product [T, 2 I]
+extern "C" int ptl_gated_act(void* out, const void* gate_up, int T_, int I, int act, float limit, int dtype,
+                             hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (I <= 0) return PTL_ERR_ARG;
+  const size_t total = (size_t)T_ * I;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == PTL_DTYPE_F32)
+    gated_act_kernel<float><<<(int)blocks, 256, 0, st>>>((float*)out, (const float*)gate_up, I, total, act, limit);
+  else if (dtype == PTL_DTYPE_BF16)
+    gated_act_kernel<bf16_t><<<(int)blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)gate_up, I, total, act, limit);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}

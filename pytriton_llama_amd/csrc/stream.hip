@@ -1,0 +1,211 @@
+// A residual stream that is kept in float32 whatever the engine's dtype, and the norms that read
+// and feed it:
+//
+//   Dynamic Tanh          y = tanh(alpha * x) * w + b            (no mean, no variance)
+//   RMS norm              y = x * rsqrt(mean(x^2) + eps) * w
+//
+// ptl_stream_add_dyt: stream += post(y) and out = pre(stream) in one pass over the rows: the norm
+//   behind a sublayer, the residual sum and the norm in front of the next sublayer. Every piece
+//   is optional: no y (only the norm in front), no post norm (a plain sum), no out, and a copy
+//   of the new stream in the engine's dtype for a product that reads the stream itself.
+// ptl_stream_add_rmsnorm: stream += rmsnorm(y) * w, the same with a norm that needs the row.
+// ptl_dyt: the norm alone, for rows that are no stream (the rows picked for the head).
+// ptl_embedding_scaled: stream[t] = table[ids[t]] * scale, in float32.
+// ptl_gelu_gather_mul: out[t, j] = gelu_tanh(z[t, j]) * table[ids[t], col0 + j]: a gate on a
+//   per-token vector looked up in a table that several layers share.
+//
+// All arithmetic is float32; tanhf / expf are the accurate ones.
+#include "common.h"
+#include <math.h>
+
+struct DytArgs {
+  const float* w;     // [H]; null: the norm is absent
+  const float* b;     // [H] or null
+  float alpha;
+};
+
+__device__ __forceinline__ float dyt_apply(const DytArgs& n, float x, int c) {
+  const float y = tanhf(n.alpha * x) * n.w[c];
+  return n.b ? y + n.b[c] : y;
+}
+
+template <typename TY, typename TO>
+__global__ void __launch_bounds__(256)
+stream_add_dyt_kernel(float* __restrict__ stream, const TY* __restrict__ y, DytArgs post,
+                      TO* __restrict__ out, DytArgs pre, TO* __restrict__ copy, size_t total, int H) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * 256;
+  for (; i < total; i += step) {
+    const int c = (int)(i % H);
+    float s = stream[i];
+    if (y) {
+      const float v = to_float<TY>(y[i]);
+      s += post.w ? dyt_apply(post, v, c) : v;
+      stream[i] = s;
+    }
+    if (out) out[i] = from_float<TO>(dyt_apply(pre, s, c));
+    if (copy) copy[i] = from_float<TO>(s);
+  }
+}
+
+template <typename TY, typename TO>
+static int launch_add_dyt(float* stream, const void* y, DytArgs post, void* out, DytArgs pre, void* copy,
+                          size_t total, int H, hipStream_t st) {
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  stream_add_dyt_kernel<TY, TO><<<(int)blocks, 256, 0, st>>>(stream, (const TY*)y, post, (TO*)out, pre,
+                                                            (TO*)copy, total, H);
+  return ptl_launch_status();
+}
+
+// y_dtype: of y; out_dtype: of out and copy. Null pointers switch the pieces off (see above).
+extern "C" int ptl_stream_add_dyt(float* stream, const void* y, int y_dtype, const float* post_w,
+                                  const float* post_b, float post_alpha, void* out, int out_dtype,
+                                  const float* pre_w, const float* pre_b, float pre_alpha, void* copy,
+                                  int T_, int H, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || !stream || (out && !pre_w)) return PTL_ERR_ARG;
+  const DytArgs post{post_w, post_b, post_alpha}, pre{pre_w, pre_b, pre_alpha};
+  const size_t total = (size_t)T_ * H;
+#define GO(TY, TO) return launch_add_dyt<TY, TO>(stream, y, post, out, pre, copy, total, H, st)
+  if (y_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_F32) GO(float, float);
+  if (y_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_BF16) GO(float, bf16_t);
+  if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_BF16) GO(bf16_t, bf16_t);
+  if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_F32) GO(bf16_t, float);
+#undef GO
+  return PTL_ERR_ARG;
+}
+
+template <typename TX, typename TO>
+__global__ void __launch_bounds__(256)
+dyt_kernel(TO* __restrict__ out, const TX* __restrict__ x, DytArgs n, size_t total, int H) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * 256;
+  for (; i < total; i += step) out[i] = from_float<TO>(dyt_apply(n, to_float<TX>(x[i]), (int)(i % H)));
+}
+
+extern "C" int ptl_dyt(void* out, int out_dtype, const void* x, int x_dtype, const float* w,
+                       const float* b, float alpha, int T_, int H, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || !w) return PTL_ERR_ARG;
+  const DytArgs n{w, b, alpha};
+  const size_t total = (size_t)T_ * H;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+#define GO(TX, TO)                                                                                   \
+  {                                                                                                  \
+    dyt_kernel<TX, TO><<<(int)blocks, 256, 0, st>>>((TO*)out, (const TX*)x, n, total, H);            \
+    return ptl_launch_status();                                                                      \
+  }
+  if (x_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_F32) GO(float, float);
+  if (x_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_BF16) GO(float, bf16_t);
+  if (x_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_BF16) GO(bf16_t, bf16_t);
+  if (x_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_F32) GO(bf16_t, float);
+#undef GO
+  return PTL_ERR_ARG;
+}
+
+// One workgroup a row: the sum of squares of y, then stream += y * rsqrt(mean + eps) * w and, when
+// asked for, out = pre(stream) and the copy of the new stream.
+template <typename TY, typename TO>
+__global__ void __launch_bounds__(256)
+stream_add_rmsnorm_kernel(float* __restrict__ stream, const TY* __restrict__ y, const float* __restrict__ w,
+                          float eps, TO* __restrict__ out, DytArgs pre, TO* __restrict__ copy, int H) {
+  __shared__ float scratch[16];
+  const size_t row = (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < H; c += 256) {
+    const float v = to_float<TY>(y[row + c]);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += 256) {
+    const float s = stream[row + c] + to_float<TY>(y[row + c]) * r * w[c];
+    stream[row + c] = s;
+    if (out) out[row + c] = from_float<TO>(dyt_apply(pre, s, c));
+    if (copy) copy[row + c] = from_float<TO>(s);
+  }
+}
+
+extern "C" int ptl_stream_add_rmsnorm(float* stream, const void* y, int y_dtype, const float* w, float eps,
+                                      void* out, int out_dtype, const float* pre_w, const float* pre_b,
+                                      float pre_alpha, void* copy, int T_, int H, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || !stream || !y || !w || (out && !pre_w)) return PTL_ERR_ARG;
+  const DytArgs pre{pre_w, pre_b, pre_alpha};
+#define GO(TY, TO)                                                                                   \
+  {                                                                                                  \
+    stream_add_rmsnorm_kernel<TY, TO><<<T_, 256, 0, st>>>(stream, (const TY*)y, w, eps, (TO*)out, pre, \
+                                                          (TO*)copy, H);                             \
+    return ptl_launch_status();                                                                      \
+  }
+  if (y_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_F32) GO(float, float);
+  if (y_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_BF16) GO(float, bf16_t);
+  if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_BF16) GO(bf16_t, bf16_t);
+  if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_F32) GO(bf16_t, float);
+#undef GO
+  return PTL_ERR_ARG;
+}
+
+template <typename T>
+__global__ void embedding_scaled_kernel(float* __restrict__ out, const T* __restrict__ table,
+                                        const int32_t* __restrict__ ids, int H, int V, float scale) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  if (id < 0 || id >= V) id = 0;          // checked on the host; never read out of bounds
+  const T* src = table + (size_t)id * H;
+  float* dst = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_float<T>(src[i]) * scale;
+}
+
+extern "C" int ptl_embedding_scaled(float* out, const void* table, const int32_t* ids, int T_, int H,
+                                    int V, float scale, int dtype, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || V <= 0) return PTL_ERR_ARG;
+  const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+  if (dtype == PTL_DTYPE_F32)
+    embedding_scaled_kernel<float><<<T_, threads, 0, st>>>(out, (const float*)table, ids, H, V, scale);
+  else if (dtype == PTL_DTYPE_BF16)
+    embedding_scaled_kernel<bf16_t><<<T_, threads, 0, st>>>(out, (const bf16_t*)table, ids, H, V, scale);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}
+
+__device__ __forceinline__ float gelu_tanh(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+gelu_gather_mul_kernel(T* __restrict__ out, const T* __restrict__ z, const T* __restrict__ table,
+                       const int32_t* __restrict__ ids, int n, int ld, int col0, int V, size_t total) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / n;
+  const int j = (int)(i - t * n);
+  int id = ids[t];
+  if (id < 0 || id >= V) id = 0;
+  const float e = to_float<T>(table[(size_t)id * ld + col0 + j]);
+  out[i] = from_float<T>(gelu_tanh(to_float<T>(z[i])) * e);
+}
+
+// z, out [T, n] dense; table [V, ld]; the token's vector is table[id, col0 : col0 + n]
+extern "C" int ptl_gelu_gather_mul(void* out, const void* z, const void* table, const int32_t* ids,
+                                   int T_, int n, int ld, int col0, int V, int dtype, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (n <= 0 || V <= 0 || col0 < 0 || col0 + n > ld) return PTL_ERR_ARG;
+  const size_t total = (size_t)T_ * n;
+  const size_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffff) return PTL_ERR_ARG;
+  if (dtype == PTL_DTYPE_F32)
+    gelu_gather_mul_kernel<float><<<(int)blocks, 256, 0, st>>>((float*)out, (const float*)z,
+                                                               (const float*)table, ids, n, ld, col0, V, total);
+  else if (dtype == PTL_DTYPE_BF16)
+    gelu_gather_mul_kernel<bf16_t><<<(int)blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)z,
+                                                                (const bf16_t*)table, ids, n, ld, col0, V, total);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}

@@ -1,2 +1,3 @@
 from .causal_lm import CausalLM, LayerCall
 from .llama import build_block, build_llama, llama_layer_specs
+from .rubasun import build_rubasun

@@ -6,4 +6,7 @@ from .kernels import (PROBE_MFMA_FLOPS_PER_ITER, ROWS_MIN, KernelError, RowScale
                       gemm_library, gemm_library_fits, timed_library_products, library_product_choice, gemm_nt, gemm_rows, gemm_rows_add_rmsnorm, gemm_rows_add_rmsnorm_fits, gemm_rows_fits, gemm_rows_splits, sum_add_rmsnorm, gemm_skinny, gemm_skinny_add_norm, gemm_skinny_add_norm_fits,
                       gemm_skinny_fits, probe_mfma, probe_stream_read, qkv_rope_store, qkv_rope_store_fits,
                       rope_store, row_scale,
-                      sample_top_p, silu_mul, stage_step, to_device, token_logprob)
+                      sample_top_p, silu_mul, stage_step, to_device, token_logprob,
+                      ACT_CLAMPED, ACT_SILU, Routing, dyt, embedding_scaled, gated_act, gelu_gather_mul,
+                      gemm_heads_nt, latent_prepare, moe_experts, moe_route, stream_add_dyt,
+                      stream_add_rmsnorm)

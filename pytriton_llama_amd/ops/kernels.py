@@ -910,3 +910,284 @@ def probe_mfma(iters: int, blocks: int, device="cuda") -> None:
     out = torch.empty(blocks * 256, dtype=torch.float32, device=device)
     lib = library.load("probe")
     _check(lib.ptl_probe_mfma(_ptr(out), int(iters), int(blocks), _stream()), "probe_mfma")
+
+
+# ---------------------------------------------------------------------------
+# The float32 residual stream and its norms (csrc/stream.hip)
+def _norm_args(norm):
+    """(weight, bias, alpha) of a Dynamic-Tanh norm as kernel arguments; ``norm``: a tuple
+    (weight float32 [H], bias float32 [H] or None, alpha) or None."""
+    if norm is None:
+        return ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_float(0.0)
+    w, b, alpha = norm
+    return _ptr(w), _ptr(b), ctypes.c_float(alpha)
+
+
+def _check_norm(norm, H: int, what: str) -> None:
+    if norm is None:
+        return
+    w, b, _ = norm
+    _need_gpu(w, b)
+    for t in (w, b):
+        if t is not None and (t.dtype != torch.float32 or t.shape != (H,) or not t.is_contiguous()):
+            raise KernelError(f"{what}: norm weight and bias must be float32 [{H}]")
+
+
+def _check_stream(stream: torch.Tensor, what: str):
+    _need_gpu(stream)
+    if stream.dim() != 2 or stream.dtype != torch.float32 or not stream.is_contiguous():
+        raise KernelError(f"{what}: the residual stream must be a contiguous float32 [T, H] matrix")
+    return stream.shape
+
+
+def embedding_scaled(table: torch.Tensor, ids: torch.Tensor, scale: float) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale as float32 (the start of a float32 residual stream)."""
+    _need_gpu(table, ids)
+    _i32(ids, "ids")
+    if table.dim() != 2 or not table.is_contiguous():
+        raise KernelError("embedding table must be a contiguous [V, H] matrix")
+    V, H = table.shape
+    T = ids.numel()
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _check(library.load("stream").ptl_embedding_scaled(_ptr(out), _ptr(table), _ptr(ids), T, H, V,
+                                                       ctypes.c_float(scale), _dtype_code(table), _stream()),
+           "embedding_scaled")
+    return out
+
+
+def dyt(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], alpha: float,
+        out_dtype: torch.dtype) -> torch.Tensor:
+    """tanh(alpha x) * weight + bias for rows x [T, H] of float32 or bfloat16."""
+    _need_gpu(x)
+    if x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("dyt: x must be a contiguous [T, H] matrix")
+    T, H = x.shape
+    _check_norm((weight, bias, alpha), H, "dyt")
+    out = torch.empty((T, H), dtype=out_dtype, device=x.device)
+    _check(library.load("stream").ptl_dyt(_ptr(out), _dtype_code(out), _ptr(x), _dtype_code(x), _ptr(weight),
+                                          _ptr(bias), ctypes.c_float(alpha), T, H, _stream()), "dyt")
+    return out
+
+
+def stream_add_dyt(stream: torch.Tensor, y: Optional[torch.Tensor], post=None, pre=None,
+                   out_dtype: Optional[torch.dtype] = None, want_copy: bool = False):
+    """stream += post(y) (plain sum when ``post`` is None, nothing when ``y`` is None), in place;
+    returns (pre(stream) in ``out_dtype`` or None, a copy of the new stream in ``out_dtype`` or
+    None). ``post`` / ``pre``: (weight, bias, alpha) of Dynamic-Tanh norms."""
+    T, H = _check_stream(stream, "stream_add_dyt")
+    if y is not None:
+        _need_gpu(y)
+        if y.shape != stream.shape or not y.is_contiguous():
+            raise KernelError("stream_add_dyt: y must be a contiguous matrix of the stream's shape")
+    _check_norm(post, H, "stream_add_dyt")
+    _check_norm(pre, H, "stream_add_dyt")
+    out_dtype = out_dtype or torch.float32
+    out = torch.empty((T, H), dtype=out_dtype, device=stream.device) if pre is not None else None
+    copy = torch.empty((T, H), dtype=out_dtype, device=stream.device) if want_copy else None
+    pw, pb, pa = _norm_args(post)
+    qw, qb, qa = _norm_args(pre)
+    code = _F32 if out_dtype == torch.float32 else _BF16
+    _check(library.load("stream").ptl_stream_add_dyt(
+        _ptr(stream), _ptr(y), _dtype_code(y) if y is not None else _F32, pw, pb, pa, _ptr(out), code,
+        qw, qb, qa, _ptr(copy), T, H, _stream()), "stream_add_dyt")
+    return out, copy
+
+
+def stream_add_rmsnorm(stream: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, pre=None,
+                       out_dtype: Optional[torch.dtype] = None, want_copy: bool = False):
+    """stream += y * rsqrt(mean(y^2) + eps) * weight, in place; returns (pre(stream) or None, a
+    copy of the new stream or None) as stream_add_dyt does."""
+    T, H = _check_stream(stream, "stream_add_rmsnorm")
+    _need_gpu(y, weight)
+    if y.shape != stream.shape or not y.is_contiguous():
+        raise KernelError("stream_add_rmsnorm: y must be a contiguous matrix of the stream's shape")
+    if weight.dtype != torch.float32 or weight.shape != (H,) or not weight.is_contiguous():
+        raise KernelError(f"stream_add_rmsnorm: weight must be float32 [{H}]")
+    _check_norm(pre, H, "stream_add_rmsnorm")
+    out_dtype = out_dtype or torch.float32
+    out = torch.empty((T, H), dtype=out_dtype, device=stream.device) if pre is not None else None
+    copy = torch.empty((T, H), dtype=out_dtype, device=stream.device) if want_copy else None
+    qw, qb, qa = _norm_args(pre)
+    code = _F32 if out_dtype == torch.float32 else _BF16
+    _check(library.load("stream").ptl_stream_add_rmsnorm(
+        _ptr(stream), _ptr(y), _dtype_code(y), _ptr(weight), ctypes.c_float(eps), _ptr(out), code, qw, qb, qa,
+        _ptr(copy), T, H, _stream()), "stream_add_rmsnorm")
+    return out, copy
+
+
+def gelu_gather_mul(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0: int) -> torch.Tensor:
+    """out[t, j] = gelu_tanh(z[t, j]) * table[ids[t], col0 + j] for z [T, n]."""
+    _need_gpu(z, table, ids)
+    _i32(ids, "ids")
+    if z.dim() != 2 or not z.is_contiguous() or table.dim() != 2 or not table.is_contiguous() \
+            or table.dtype != z.dtype:
+        raise KernelError("gelu_gather_mul: z [T, n] and table [V, ld] must be contiguous and of one dtype")
+    T, n = z.shape
+    V, ld = table.shape
+    if ids.numel() != T or col0 < 0 or col0 + n > ld:
+        raise KernelError("gelu_gather_mul: one id per row, and the columns must lie inside the table")
+    out = torch.empty_like(z)
+    _check(library.load("stream").ptl_gelu_gather_mul(_ptr(out), _ptr(z), _ptr(table), _ptr(ids), T, n, ld,
+                                                      int(col0), V, _dtype_code(z), _stream()),
+           "gelu_gather_mul")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Latent attention (csrc/latent.hip)
+def latent_prepare(q_out: torch.Tensor, proj: torch.Tensor, q_off: int, kv_off: int,
+                   positions: torch.Tensor, inv_freq: Optional[torch.Tensor], c_weight: Optional[torch.Tensor],
+                   eps: float, slots: Optional[torch.Tensor], cache: Optional[torch.Tensor],
+                   H: int, dn: int, dr: int, R: int) -> None:
+    """From the projections ``proj`` [T, >= q_off + H (dn + dr)] of a step: the rotated query
+    parts into q_out[:, :, R:] (q_out [T, H, R + dr]), and, when the layer has a down-projection
+    (``kv_off`` >= 0: its R + dr columns start there) and ``slots`` are given, the normalised
+    latent and the rotated shared key part into ``cache`` [pages, 1, page_size, R + dr] at the
+    tokens' slots. inv_freq float32 [pairs], 2 * pairs <= dr: the entries that rotate."""
+    _need_gpu(q_out, proj, positions, inv_freq, c_weight, slots, cache)
+    T = proj.shape[0]
+    D = R + dr
+    if proj.dim() != 2 or proj.stride(1) != 1 or q_out.shape != (T, H, D) or not q_out.is_contiguous() \
+            or q_out.dtype != proj.dtype:
+        raise KernelError("latent_prepare: proj [T, n] with dense rows, q_out contiguous [T, H, R + dr]")
+    if q_off < 0 or q_off + H * (dn + dr) > proj.shape[1] or (kv_off >= 0 and kv_off + D > proj.shape[1]):
+        raise KernelError("latent_prepare: the columns named lie outside the projections")
+    _i32(positions, "positions")
+    if positions.numel() != T or dr % 2:
+        raise KernelError("latent_prepare: one position per token, an even rotated size")
+    pairs = 0
+    if inv_freq is not None:
+        pairs = inv_freq.numel()
+        if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous() or 2 * pairs > dr:
+            raise KernelError("latent_prepare: inv_freq must be float32 with at most dr / 2 entries")
+    if kv_off >= 0 and slots is not None:
+        _i32(slots, "slots")
+        if slots.numel() != T:
+            raise KernelError("latent_prepare: one slot per token")
+        if cache is None or cache.dim() != 4 or cache.shape[1] != 1 or cache.shape[3] != D \
+                or cache.dtype != proj.dtype or not cache.is_contiguous():
+            raise KernelError(f"latent_prepare: cache must be contiguous [pages, 1, page_size, {D}]")
+        if c_weight is None or c_weight.dtype != torch.float32 or c_weight.shape != (R,) \
+                or not c_weight.is_contiguous():
+            raise KernelError(f"latent_prepare: the latent's norm weight must be float32 [{R}]")
+    _check(library.load("latent").ptl_latent_prepare(
+        _ptr(q_out), ctypes.c_long(H * D), _ptr(proj), ctypes.c_long(proj.stride(0)), int(q_off), int(kv_off),
+        _ptr(positions), _ptr(inv_freq), int(pairs), _ptr(c_weight), ctypes.c_float(eps), _ptr(slots),
+        _ptr(cache), T, H, dn, dr, R, _dtype_code(proj), _stream()), "latent_prepare")
+
+
+def gemm_heads_nt(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor,
+                  gate: Optional[torch.Tensor] = None) -> None:
+    """out[t, h, :] = x[t, h, :] @ w[h].T for views out [T, H, N], x [T, H, K] (dense last
+    dimension, any row and head strides) and w [H, N, K] contiguous; ``gate`` [T, H] (a view
+    with stride 1 over the heads): the result of head h of row t times sigmoid(gate[t, h])."""
+    _need_gpu(out, x, w, gate)
+    if x.dim() != 3 or out.dim() != 3 or w.dim() != 3 or not w.is_contiguous():
+        raise KernelError("gemm_heads_nt: x [T, H, K], out [T, H, N], w contiguous [H, N, K]")
+    T, H, K = x.shape
+    N = w.shape[1]
+    if w.shape != (H, N, K) or out.shape != (T, H, N) or x.stride(2) != 1 or out.stride(2) != 1:
+        raise KernelError("gemm_heads_nt: shapes do not match, or a last dimension is not dense")
+    if not (x.dtype == out.dtype == w.dtype):
+        raise KernelError("gemm_heads_nt: one dtype")
+    ldg = 0
+    if gate is not None:
+        if gate.shape != (T, H) or gate.dtype != x.dtype or (H > 1 and gate.stride(1) != 1):
+            raise KernelError("gemm_heads_nt: gate must be [T, H] with dense rows")
+        ldg = gate.stride(0)
+    _check(library.load("latent").ptl_gemm_heads_nt(
+        _ptr(out), ctypes.c_long(out.stride(0)), ctypes.c_long(out.stride(1)), _ptr(x),
+        ctypes.c_long(x.stride(0)), ctypes.c_long(x.stride(1)), _ptr(w), T, H, N, K, _ptr(gate),
+        ctypes.c_long(ldg), _dtype_code(x), _stream()), "gemm_heads_nt")
+
+
+# ---------------------------------------------------------------------------
+# Routed experts (csrc/moe.hip)
+ACT_SILU, ACT_CLAMPED = 0, 1
+
+
+def gated_act(gate_up: torch.Tensor, act: int, limit: float = 0.0) -> torch.Tensor:
+    """The gated activation ``act`` on a dense gate|up product [T, 2 I] -> [T, I]."""
+    _need_gpu(gate_up)
+    if gate_up.dim() != 2 or not gate_up.is_contiguous() or gate_up.shape[1] % 2:
+        raise KernelError("gated_act: input must be a contiguous [T, 2I] matrix")
+    T, I2 = gate_up.shape
+    out = torch.empty((T, I2 // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _check(library.load("moe").ptl_gated_act(_ptr(out), _ptr(gate_up), T, I2 // 2, int(act),
+                                             ctypes.c_float(limit), _dtype_code(gate_up), _stream()), "gated_act")
+    return out
+
+
+class Routing:
+    """Where the (token, choice) pairs of a step went: see csrc/moe.hip."""
+    __slots__ = ("idx", "wgt", "extra", "pos_of", "sorted", "expert_end", "tile_expert", "tile_row0",
+                 "max_tiles", "top", "experts")
+
+
+def moe_route(logits: torch.Tensor, experts: int, top: int, extra: int = 0,
+              renormalize: bool = False) -> Routing:
+    """Route every row of float32 ``logits`` [T, experts + extra] to its ``top`` experts by the
+    sigmoid of its logits and order the pairs by expert."""
+    _need_gpu(logits)
+    if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1 \
+            or logits.shape[1] < experts + extra:
+        raise KernelError("moe_route: logits must be float32 [T, experts + extra] with dense rows")
+    if not 0 < top <= experts or experts > 1024 or not 0 <= extra <= 64:
+        raise KernelError(f"moe_route: {top} of {experts} experts (+{extra}) is not a case the kernel takes")
+    T = logits.shape[0]
+    A = T * top
+    lib = library.load("moe")
+    r = Routing()
+    r.top, r.experts = top, experts
+    dev = logits.device
+    r.max_tiles = int(lib.ptl_moe_max_tiles(A, experts))
+    ints = torch.empty(3 * A + experts + 2 * r.max_tiles, dtype=torch.int32, device=dev)
+    r.idx, r.pos_of, r.sorted = ints[:A], ints[A:2 * A], ints[2 * A:3 * A]
+    r.expert_end = ints[3 * A:3 * A + experts]
+    r.tile_expert = ints[3 * A + experts:3 * A + experts + r.max_tiles]
+    r.tile_row0 = ints[3 * A + experts + r.max_tiles:]
+    r.wgt = torch.empty(A, dtype=torch.float32, device=dev)
+    r.extra = torch.empty((T, extra), dtype=torch.float32, device=dev) if extra else None
+    _check(lib.ptl_moe_topk(_ptr(logits), int(logits.stride(0)), T, experts, top, extra, int(renormalize),
+                            _ptr(r.idx), _ptr(r.wgt), _ptr(r.extra), _stream()), "moe_topk")
+    _check(lib.ptl_moe_sort(_ptr(r.idx), A, experts, _ptr(r.pos_of), _ptr(r.sorted), _ptr(r.expert_end),
+                            _ptr(r.tile_expert), _ptr(r.tile_row0), r.max_tiles, _stream()), "moe_sort")
+    return r
+
+
+def moe_experts(x: torch.Tensor, r: Routing, gate_up: torch.Tensor, down: torch.Tensor, act: int,
+                limit: float, weight_on_input: bool, shared: Optional[torch.Tensor] = None,
+                shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The routed experts on x [T, K]: gate_up [E, 2 I, K], down [E, N, I]; returns float32
+    [T, N] = sum over a row's choices of its experts' outputs (+ shared_gate[t] * shared[t])."""
+    _need_gpu(x, gate_up, down, shared, shared_gate)
+    T, K = x.shape
+    E, I2, _ = gate_up.shape
+    I, N = I2 // 2, down.shape[1]
+    if x.stride(1) != 1 or gate_up.shape != (E, 2 * I, K) or down.shape != (E, N, I) or E != r.experts \
+            or not gate_up.is_contiguous() or not down.is_contiguous() \
+            or not (x.dtype == gate_up.dtype == down.dtype) or r.idx.numel() != T * r.top:
+        raise KernelError("moe_experts: shapes or dtypes do not fit the routing")
+    if shared is not None and (shared.shape != (T, N) or shared.dtype != x.dtype or not shared.is_contiguous()):
+        raise KernelError("moe_experts: the shared expert's output must be contiguous [T, N]")
+    if shared_gate is not None and (shared_gate.dtype != torch.float32 or shared_gate.shape[0] != T
+                                    or shared_gate.dim() != 2):
+        raise KernelError("moe_experts: the shared expert's gate must be float32 [T, n]")
+    lib = library.load("moe")
+    A = T * r.top
+    code = _dtype_code(x)
+    mid = torch.empty((A, I), dtype=x.dtype, device=x.device)
+    _check(lib.ptl_moe_gate_up(_ptr(mid), ctypes.c_long(I), _ptr(x), ctypes.c_long(x.stride(0)), _ptr(gate_up),
+                               _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), _ptr(r.sorted),
+                               _ptr(r.wgt) if weight_on_input else None, r.max_tiles, r.top, I, K, int(act),
+                               ctypes.c_float(limit), code, _stream()), "moe_gate_up")
+    rows = torch.empty((A, N), dtype=x.dtype, device=x.device)
+    _check(lib.ptl_moe_down(_ptr(rows), ctypes.c_long(N), _ptr(mid), ctypes.c_long(I), _ptr(down),
+                            _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), r.max_tiles, N, I,
+                            code, _stream()), "moe_down")
+    y = torch.empty((T, N), dtype=torch.float32, device=x.device)
+    _check(lib.ptl_moe_combine(_ptr(y), _ptr(rows), ctypes.c_long(N), _ptr(r.pos_of),
+                               None if weight_on_input else _ptr(r.wgt), r.top, _ptr(shared), _ptr(shared_gate),
+                               int(shared_gate.stride(0)) if shared_gate is not None else 0, T, N, code,
+                               _stream()), "moe_combine")
+    return y

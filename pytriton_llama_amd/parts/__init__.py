@@ -2,9 +2,11 @@ from .base import (PART_KINDS, PART_REGISTRY, PagedSpec, PagedTensor, ParamSourc
                    build_part, paged_kv_spec,
                    place, register_part)
 from .linear import linear
-from .norm import RMSNorm
+from .norm import DynamicTanh, RMSNorm
 from .rotary import RotaryEncoding, default_inv_freq, llama3_inv_freq
 from .attention import PagedAttention
-from .feedforward import SwiGLU
+from .feedforward import GatedMLP, RoutedExperts, SwiGLU
+from .latent_attention import LatentAttention
+from .token_input import GatedTokenInput, TokenTable
 from .embedding import LinearHead, TokenEmbedding
-from .block import PreNormBlock
+from .block import PreNormBlock, SandwichBlock

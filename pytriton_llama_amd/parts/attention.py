@@ -41,8 +41,9 @@ class PagedAttention(Part):
                  v_name: str = "v_proj.weight", o_name: str = "o_proj.weight"):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
-        if head_dim % 2 or head_dim > 256:
-            raise ValueError(f"the attention kernels take even head sizes up to 256, got {head_dim}")
+        if (head_dim % 2 and position is not None) or head_dim > 256:
+            raise ValueError(f"the attention kernels take head sizes up to 256 (even ones with a "
+                             f"position encoding), got {head_dim}")
         self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
         self.num_kv_heads, self.head_dim = int(num_kv_heads), int(head_dim)
         self.position = position
@@ -166,14 +167,19 @@ class PagedAttention(Part):
             want = -(-4 * cus // base)
         return max(1, min(want, -(-span // turn), 64))
 
-    def attend(self, out, q, cache, ctx, group) -> None:
+    def attend(self, out, q, cache, ctx, group, k=None, v=None) -> None:
+        """``k`` / ``v``: the pools of keys and of values, [pages, Hkv, page_size, D] each, when
+        they are not the cache layer's "k" and "v" (a mixer that keeps one tensor a token and
+        reads it as both)."""
+        k = cache.k if k is None else k
+        v = cache.v if v is None else v
         D, window = self.head_dim, self.window or 0
         n_dec = ctx.num_decode_seqs if D % 16 == 0 else 0
         if n_dec:
             mfma = (ops.attention_decode_mfma_fits(q.dtype, self.num_heads, self.num_kv_heads, D,
                                                    cache.page_size)
                     and q.stride(0) % 8 == 0)
-            ops.attention_decode(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
+            ops.attention_decode(out, q, k, v, ctx.q_start, ctx.ctx_len,
                                  group.block_table, n_dec, self.scale, window,
                                  self.decode_splits(ctx, n_dec, mfma, q.device), matrix_cores=mfma)
         if n_dec == ctx.num_seqs:
@@ -185,10 +191,10 @@ class PagedAttention(Part):
                 q.device, self.num_heads, D, ctx.work[PORTIONS_64][0].numel(),
                 ctx.work[PORTIONS_128][0].numel(), min(keys, window) if window else keys)
             ws, wo = ctx.work[PORTIONS_128 if rows == 128 else PORTIONS_64]
-            ops.attention_prefill_mfma(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
+            ops.attention_prefill_mfma(out, q, k, v, ctx.q_start, ctx.ctx_len,
                                        group.block_table, ws, wo, self.scale, window, rows, groups)
         else:
             ws, wo = ctx.work[PORTIONS_16 if n_dec else ALL_16]
-            ops.attention_generic(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
+            ops.attention_generic(out, q, k, v, ctx.q_start, ctx.ctx_len,
                                   group.block_table, ws, wo, self.scale, window)
 

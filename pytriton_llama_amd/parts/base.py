@@ -201,7 +201,7 @@ class Part:
         return 0
 
 
-PART_KINDS = ("embedding", "norm", "mixer", "feed_forward", "position", "head", "block")
+PART_KINDS = ("embedding", "norm", "mixer", "feed_forward", "position", "head", "block", "stream_input")
 PART_REGISTRY: Dict[str, Dict[str, Any]] = {k: {} for k in PART_KINDS}
 
 

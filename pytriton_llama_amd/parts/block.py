@@ -1,6 +1,9 @@
 """Arrangements of norm, mixer and feed-forward in a block."""
 from __future__ import annotations
 
+import torch
+
+from .. import ops
 from .base import Part, as_tensor, register_part, run_norm
 
 
@@ -71,3 +74,104 @@ class PreNormBlock(Part):
         else:
             h = ffn.forward(h)
         return h, residual
+
+
+@register_part("block", "sandwich")
+class SandwichBlock(Part):
+    """A norm in front of and behind every sublayer, on a residual stream kept in float32:
+
+        x <- x + post1(mixer(pre1(x)));   x <- x + post2(ffn(pre2(x)));   x <- side(x, tokens)
+
+    The feed-forward (with its two norms) and the side input are optional. The stream is the
+    block's ``h`` (float32 [T, hidden], updated in place); ``residual`` stays None. With
+    Dynamic-Tanh norms the norm behind a sublayer, the sum and the norm in front of the next
+    one are one kernel (ops.stream_add_dyt); other norms run through their own ``forward``
+    and a plain sum into the stream. Sublayers read and return the engine's dtype (a
+    feed-forward may return float32)."""
+
+    def __init__(self, pre_mixer_norm: Part, mixer: Part, post_mixer_norm: Part,
+                 pre_ffn_norm: Part = None, feed_forward: Part = None, post_ffn_norm: Part = None,
+                 side: Part = None):
+        if (feed_forward is None) != (pre_ffn_norm is None) or (feed_forward is None) != (post_ffn_norm is None):
+            raise ValueError("a feed-forward comes with both of its norms, or none of the three")
+        self.norm1, self.mixer, self.norm1b = pre_mixer_norm, mixer, post_mixer_norm
+        self.norm2, self.feed_forward, self.norm2b = pre_ffn_norm, feed_forward, post_ffn_norm
+        self.side = side
+        libs = ("stream",)
+        for p in self.children().values():
+            libs += tuple(p.kernel_libraries)
+        self.kernel_libraries = tuple(dict.fromkeys(libs))
+        self.dtype = None
+
+    def children(self):
+        roles = {"norm1": self.norm1, "mixer": self.mixer, "norm1b": self.norm1b, "norm2": self.norm2,
+                 "feed_forward": self.feed_forward, "norm2b": self.norm2b, "side": self.side}
+        return {k: p for k, p in roles.items() if p is not None}
+
+    def cache_spec(self):
+        return self.mixer.cache_spec() if hasattr(self.mixer, "cache_spec") else None
+
+    def work_lists(self):
+        lists = ()
+        for p in self.children().values():
+            if hasattr(p, "work_lists"):
+                lists += tuple(p.work_lists())
+        return tuple(dict.fromkeys(lists))
+
+    def make_decode_copies(self) -> int:
+        return sum(p.make_decode_copies() for p in self.children().values()
+                   if hasattr(p, "make_decode_copies"))
+
+    @property
+    def graph_capturable(self) -> bool:
+        return all(getattr(p, "graph_capturable", True) for p in self.children().values())
+
+    @staticmethod
+    def _fusable(norm) -> bool:
+        return norm is None or hasattr(norm, "params")
+
+    def _add(self, stream, y, post, pre, dtype, want_copy=False):
+        """stream += post(y); returns (pre(stream) or None, copy or None)."""
+        if self._fusable(post) and self._fusable(pre):
+            return ops.stream_add_dyt(stream, y, post.params() if post is not None else None,
+                                      pre.params() if pre is not None else None, dtype, want_copy)
+        if y is not None:
+            if post is not None:
+                y = post.forward(y if y.dtype == dtype else y.to(dtype), None)[0]
+            ops.stream_add_dyt(stream, y, None, None, dtype)
+        copy = None
+        if want_copy or pre is not None:
+            _, copy = ops.stream_add_dyt(stream, None, None, None, dtype, True)
+        out = pre.forward(copy, None)[0] if pre is not None else None
+        return out, copy
+
+    def forward(self, h, residual, ctx, cache):
+        if residual is not None or h.dtype != torch.float32:
+            raise ops.KernelError("a sandwich block runs on a float32 residual stream without a second one")
+        stream = h
+        dtype = self.mixer_dtype()
+        a, _ = self._add(stream, None, None, self.norm1, dtype)
+        y = self.mixer.forward(a, ctx, cache)
+        want_copy = self.side is not None and dtype != torch.float32
+        if self.feed_forward is not None:
+            a, _ = self._add(stream, y, self.norm1b, self.norm2, dtype)
+            y = self.feed_forward.forward(a)
+            _, copy = self._add(stream, y, self.norm2b, None, dtype, want_copy)
+        else:
+            _, copy = self._add(stream, y, self.norm1b, None, dtype, want_copy)
+        if self.side is not None:
+            self.side.forward(stream, copy if want_copy else stream, ctx.token_ids)
+        return stream, None
+
+    def mixer_dtype(self):
+        """The engine's dtype, as the parts hold it after loading."""
+        if self.dtype is None:
+            self.dtype = getattr(self.norm1, "dtype", None)
+        if self.dtype is None:
+            for p in self.children().values():
+                for t in vars(p).values():
+                    if isinstance(t, torch.Tensor) and t.dim() >= 2 and t.is_floating_point():
+                        self.dtype = t.dtype
+                        return self.dtype
+            raise RuntimeError("the block's parts hold no weights yet")
+        return self.dtype

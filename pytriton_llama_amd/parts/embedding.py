@@ -12,11 +12,19 @@ from .linear import LINEAR_LIBRARIES, decode_copy, linear
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
-    """h[t] = E[ids[t]], no scaling (lite_llama/models/llama.py:179,201)."""
+    """h[t] = E[ids[t]], no scaling (lite_llama/models/llama.py:179,201). With
+    ``float32_stream`` the result is E[ids[t]] * scale in float32 whatever the engine's dtype:
+    the start of a residual stream that blocks keep in float32."""
     kernel_libraries = ("embedding",)
 
-    def __init__(self, vocab_size: int, hidden_size: int, weight_name: str = "weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, weight_name: str = "weight",
+                 scale: float = 1.0, float32_stream: bool = False):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.scale, self.float32_stream = float(scale), bool(float32_stream)
+        if self.float32_stream:
+            self.kernel_libraries = ("stream",)
+        if self.scale != 1.0 and not self.float32_stream:
+            raise ValueError("a scaled embedding is computed into a float32 stream")
         self.weight_name = weight_name
         self.weight: Optional[torch.Tensor] = None
 
@@ -27,6 +35,8 @@ class TokenEmbedding(Part):
         self.weight = place(tensors[self.weight_name], "matrix", dtype, device)
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+        if self.float32_stream:
+            return ops.embedding_scaled(self.weight, token_ids, self.scale)
         return ops.embedding(self.weight, token_ids)
 
 

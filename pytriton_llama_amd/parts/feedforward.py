@@ -61,3 +61,122 @@ class SwiGLU(Part):
         if defer_output:                    # (the norm that follows picks the kernels by the rows)
             return PendingProduct(a, self.down, self.down_blocked)
         return linear(a, self.down, blocked=self.down_blocked)
+
+
+@register_part("feed_forward", "gated_mlp")
+class GatedMLP(Part):
+    """down(act(gate(x), up(x))) with the activation as a parameter: "silu" (silu(g) * u) or
+    "clamped" (g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1)).
+    No biases. gate and up are one [2I, hidden] matrix at run time."""
+    kernel_libraries = ("moe",) + LINEAR_LIBRARIES
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu",
+                 limit: float = 0.0, gate_name: str = "gate", up_name: str = "up", down_name: str = "down"):
+        if activation not in ("silu", "clamped"):
+            raise ValueError(f"unknown gated activation {activation!r}")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.act = ops.ACT_CLAMPED if activation == "clamped" else ops.ACT_SILU
+        self.limit = float(limit)
+        self.names = (gate_name, up_name, down_name)
+        self.gate_up = self.down = self.gate_up_blocked = self.down_blocked = None
+
+    def param_sources(self) -> List[ParamSource]:
+        g, u, d = self.names
+        return [ParamSource(g, (self.intermediate_size, self.hidden_size)),
+                ParamSource(u, (self.intermediate_size, self.hidden_size)),
+                ParamSource(d, (self.hidden_size, self.intermediate_size))]
+
+    def load(self, tensors, dtype, device) -> None:
+        g, u, d = self.names
+        self.gate_up = place(torch.cat([tensors[g], tensors[u]], dim=0), "matrix", dtype, device)
+        self.down = place(tensors[d], "matrix", dtype, device)
+
+    def make_decode_copies(self) -> int:
+        self.gate_up_blocked, self.down_blocked = decode_copy(self.gate_up), decode_copy(self.down)
+        return sum(t.numel() * t.element_size() for t in (self.gate_up_blocked, self.down_blocked)
+                   if t is not None)
+
+    def forward(self, x):
+        x = as_tensor(x)
+        a = ops.gated_act(linear(x, self.gate_up, blocked=self.gate_up_blocked), self.act, self.limit)
+        return linear(a, self.down, blocked=self.down_blocked)
+
+
+@register_part("feed_forward", "routed_experts")
+class RoutedExperts(Part):
+    """A mixture of gated feed-forward experts: router logits z = W_r x in float32 (from the
+    rounded x and W_r of the engine's dtype, summed in float32), scores sigmoid(z), the ``top``
+    experts with the largest scores, their scores as weights (``renormalize``: divided by their
+    sum). ``weight_on_input``: the weight multiplies what the expert reads, y = sum_k
+    expert_k(s_k x), instead of what it returns. ``shared``: a GatedMLP that every token runs,
+    added times sigmoid(w_sg . x) when ``shared_gate``. The result is float32 (the sum over a
+    token's experts is made there). Nothing comes back to the host: routing, the grouping of
+    tokens by expert and the experts' products are kernels of csrc/moe.hip.
+
+    Checkpoint tensors: ``router`` [E, hidden], ``e<i>.gate|up|down``, and for the shared expert
+    ``shared.gate|up|down`` and ``shared.sg`` [1, hidden] (names are parameters)."""
+    kernel_libraries = ("moe",) + LINEAR_LIBRARIES
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
+                 activation: str = "clamped", limit: float = 0.0, weight_on_input: bool = True,
+                 renormalize: bool = False, shared: Optional[GatedMLP] = None, shared_gate: bool = True,
+                 router_name: str = "router", expert_prefix: str = "e", shared_prefix: str = "shared.",
+                 shared_gate_name: str = "shared.sg", gate_name: str = "gate", up_name: str = "up",
+                 down_name: str = "down"):
+        if not 0 < top <= num_experts:
+            raise ValueError(f"{top} of {num_experts} experts")
+        if activation not in ("silu", "clamped"):
+            raise ValueError(f"unknown gated activation {activation!r}")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.num_experts, self.top = int(num_experts), int(top)
+        self.act = ops.ACT_CLAMPED if activation == "clamped" else ops.ACT_SILU
+        self.limit = float(limit)
+        self.weight_on_input, self.renormalize = bool(weight_on_input), bool(renormalize)
+        self.shared = shared
+        self.shared_gate = bool(shared_gate) and shared is not None
+        self.router_name, self.expert_prefix = router_name, expert_prefix
+        self.shared_prefix, self.shared_gate_name = shared_prefix, shared_gate_name
+        self.names = (gate_name, up_name, down_name)
+        self.router = self.gate_up = self.down = None
+        if shared is not None:
+            self.kernel_libraries = tuple(dict.fromkeys(self.kernel_libraries + tuple(shared.kernel_libraries)))
+
+    def param_sources(self) -> List[ParamSource]:
+        g, u, d = self.names
+        I, W = self.intermediate_size, self.hidden_size
+        out = [ParamSource(self.router_name, (self.num_experts, W))]
+        for e in range(self.num_experts):
+            p = f"{self.expert_prefix}{e}."
+            out += [ParamSource(p + g, (I, W)), ParamSource(p + u, (I, W)), ParamSource(p + d, (W, I))]
+        if self.shared is not None:
+            for src in self.shared.param_sources():
+                out.append(ParamSource(self.shared_prefix + src.name, src.shape, src.kind, src.init))
+            if self.shared_gate:
+                out.append(ParamSource(self.shared_gate_name, (1, W)))
+        return out
+
+    def load(self, tensors, dtype, device) -> None:
+        g, u, d = self.names
+        router = [tensors[self.router_name]]
+        if self.shared_gate:
+            router.append(tensors[self.shared_gate_name])
+        self.router = place(torch.cat(router, dim=0), "matrix", dtype, device)
+        names = [f"{self.expert_prefix}{e}." for e in range(self.num_experts)]
+        self.gate_up = place(torch.stack([torch.cat([tensors[p + g], tensors[p + u]], dim=0) for p in names]),
+                             "matrix", dtype, device)
+        self.down = place(torch.stack([tensors[p + d] for p in names]), "matrix", dtype, device)
+        if self.shared is not None:
+            n = len(self.shared_prefix)
+            self.shared.load({k[n:]: t for k, t in tensors.items()
+                              if k.startswith(self.shared_prefix) and k != self.shared_gate_name}, dtype, device)
+
+    def make_decode_copies(self) -> int:
+        return self.shared.make_decode_copies() if self.shared is not None else 0
+
+    def forward(self, x):
+        x = as_tensor(x)
+        logits = linear(x, self.router, out_dtype=torch.float32)
+        r = ops.moe_route(logits, self.num_experts, self.top, 1 if self.shared_gate else 0, self.renormalize)
+        shared = self.shared.forward(x) if self.shared is not None else None
+        return ops.moe_experts(x, r, self.gate_up, self.down, self.act, self.limit, self.weight_on_input,
+                               shared, r.extra)

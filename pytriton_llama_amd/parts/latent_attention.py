@@ -1,0 +1,147 @@
+"""Attention over a compressed (latent) cache that all heads share."""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from .attention import PagedAttention
+from .base import PagedSpec, PagedTensor, ParamSource, Part, as_tensor, place, register_part
+from .linear import LINEAR_LIBRARIES, decode_copy, linear
+
+
+def paired_inv_freq(base: float, dims: int) -> torch.Tensor:
+    """f_i = base^(-2i / dims), i < dims / 2, for rotations of neighbouring pairs (2i, 2i + 1)."""
+    i = torch.arange(0, dims // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / dims)).to(torch.float32)
+
+
+@register_part("mixer", "latent_attention")
+class LatentAttention(Part):
+    """Causal softmax attention whose cache holds, per token, one latent vector c [kv_rank]
+    (a down-projection of the input, RMS-normed) and one rotated key part kr [rot_dim]; every
+    head's keys and values are linear maps of c:
+
+        q_h = [qn_h | qr_h] = W_q x            qn_h [dim], qr_h [rot_dim] (rotated)
+        score_h(i, j) = (qn_h(i) . Uk_h c_j + qr_h(i) . kr_j) * scale,  j <= i
+        out = W_o concat_h( sigmoid(w_g,h . x) * Uv_h sum_j p_h(i, j) c_j )
+
+    The maps move to the query side (q'_h = [Uk_h^T qn_h | qr_h], values c_j), so the attention
+    kernels read the cache as it lies: one kv head of size kv_rank + rot_dim whose keys and
+    values are the same pages (csrc/latent.hip). The rotation turns neighbouring pairs of the
+    first ``rot_dims`` entries of the rotated part by position * rot_base^(-2i / rot_dims).
+
+    ``own_kv`` False: the layer has no down-projection and reads the cache layer another one
+    fills (the model's run order hands it that layer, not writable); its kv_rank, rot_dim and
+    rotation are the owner's. ``gated`` False: no output gate. Tensor names are parameters."""
+
+    def __init__(self, hidden_size: int, num_heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
+                 scale: float, rot_base: float, rot_dims: Optional[int] = None, eps: float = 1e-6,
+                 own_kv: bool = True, gated: bool = True,
+                 q_name: str = "q", dkv_name: str = "dkv", c_norm_name: str = "dkv.norm",
+                 uk_name: str = "uk", uv_name: str = "uv", g_name: str = "g", o_name: str = "o"):
+        rot_dims = rot_dim if rot_dims is None else int(rot_dims)
+        if rot_dim % 2 or rot_dims % 2 or rot_dims > rot_dim:
+            raise ValueError(f"rotated size {rot_dim} with {rot_dims} rotating entries: both must be even, "
+                             "the second at most the first")
+        if kv_rank + rot_dim > 256:
+            raise ValueError(f"the attention kernels take kv_rank + rot_dim up to 256, got {kv_rank + rot_dim}")
+        self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
+        self.dim, self.rot_dim, self.vdim, self.kv_rank = int(dim), int(rot_dim), int(vdim), int(kv_rank)
+        self.scale, self.eps = float(scale), float(eps)
+        self.own_kv, self.gated = bool(own_kv), bool(gated)
+        self.inv_freq_host = paired_inv_freq(rot_base, rot_dims) if rot_dims else None
+        self.inv_freq: Optional[torch.Tensor] = None
+        self.names = dict(q=q_name, dkv=dkv_name, c_norm=c_norm_name, uk=uk_name, uv=uv_name, g=g_name, o=o_name)
+        D = self.kv_rank + self.rot_dim
+        # the attention itself: the engine's paged attention with one kv head of size D whose
+        # keys and values are the same pool
+        self.core = PagedAttention(hidden_size, num_heads, 1, D, position=None, scale=self.scale)
+        self.q_size = self.num_heads * (self.dim + self.rot_dim)
+        self.kv_off = self.q_size if self.own_kv else -1
+        self.g_off = self.q_size + (D if self.own_kv else 0)
+        self.proj: Optional[torch.Tensor] = None          # rows q | down-projection | gate
+        self.ukT: Optional[torch.Tensor] = None           # [H, kv_rank, dim]
+        self.uv: Optional[torch.Tensor] = None            # [H, vdim, kv_rank]
+        self.o: Optional[torch.Tensor] = None
+        self.c_weight: Optional[torch.Tensor] = None
+        self.proj_blocked = self.o_blocked = None
+        libs = ("latent",) + tuple(self.core.kernel_libraries)
+        self.kernel_libraries = tuple(dict.fromkeys(l for l in libs if l != "rope"))
+
+    @property
+    def force_decode_splits(self) -> int:
+        return self.core.force_decode_splits
+
+    @force_decode_splits.setter
+    def force_decode_splits(self, n: int) -> None:
+        self.core.force_decode_splits = n
+
+    def work_lists(self):
+        return self.core.work_lists()
+
+    def cache_spec(self):
+        """One tensor a token, [c | kr]; pages [1, page_size, kv_rank + rot_dim]. A layer
+        without a down-projection keeps nothing of its own."""
+        if not self.own_kv:
+            return None
+        return PagedSpec((PagedTensor("latent", (1, self.kv_rank + self.rot_dim), 1),), None)
+
+    def param_sources(self) -> List[ParamSource]:
+        n, H, W = self.names, self.num_heads, self.hidden_size
+        out = [ParamSource(n["q"], (self.q_size, W))]
+        if self.own_kv:
+            out += [ParamSource(n["dkv"], (self.kv_rank + self.rot_dim, W)),
+                    ParamSource(n["c_norm"], (self.kv_rank,), "vector")]
+        out += [ParamSource(n["uk"], (H * self.dim, self.kv_rank)),
+                ParamSource(n["uv"], (H * self.vdim, self.kv_rank))]
+        if self.gated:
+            out.append(ParamSource(n["g"], (H, W)))
+        out.append(ParamSource(n["o"], (W, H * self.vdim)))
+        return out
+
+    def load(self, tensors, dtype, device) -> None:
+        n, H = self.names, self.num_heads
+        rows = [tensors[n["q"]]]
+        if self.own_kv:
+            rows.append(tensors[n["dkv"]])
+            self.c_weight = place(tensors[n["c_norm"]], "vector", dtype, device)
+        if self.gated:
+            rows.append(tensors[n["g"]])
+        rows = torch.cat(rows, dim=0)
+        pad = -rows.shape[0] % 8            # (rows of the result stay 16-byte aligned in bfloat16)
+        if pad:
+            rows = torch.cat([rows, rows.new_zeros((pad, rows.shape[1]))], dim=0)
+        self.proj = place(rows, "matrix", dtype, device)
+        uk = tensors[n["uk"]].view(H, self.dim, self.kv_rank)
+        self.ukT = place(uk.transpose(1, 2), "matrix", dtype, device)
+        self.uv = place(tensors[n["uv"]].view(H, self.vdim, self.kv_rank), "matrix", dtype, device)
+        self.o = place(tensors[n["o"]], "matrix", dtype, device)
+        if self.inv_freq_host is not None:
+            self.inv_freq = self.inv_freq_host.to(device)
+
+    def make_decode_copies(self) -> int:
+        self.proj_blocked, self.o_blocked = decode_copy(self.proj), decode_copy(self.o)
+        return sum(t.numel() * t.element_size() for t in (self.proj_blocked, self.o_blocked)
+                   if t is not None)
+
+    def forward(self, x, ctx, cache):
+        x = as_tensor(x)
+        T, H, R, dr = x.shape[0], self.num_heads, self.kv_rank, self.rot_dim
+        D = R + dr
+        group = ctx.groups[cache.group]
+        pool = cache.tensors["latent"]
+        p = linear(x, self.proj, blocked=self.proj_blocked)
+        q = torch.empty((T, H, D), dtype=x.dtype, device=x.device)
+        ops.latent_prepare(q, p, 0, self.kv_off, ctx.positions, self.inv_freq, self.c_weight, self.eps,
+                           group.slots if (cache.writable and self.own_kv) else None, pool,
+                           H, self.dim, dr, R)
+        qn = p[:, :self.q_size].view(T, H, self.dim + dr)[:, :, :self.dim]
+        ops.gemm_heads_nt(q[:, :, :R], qn, self.ukT)
+        lat = torch.empty((T, H, D), dtype=x.dtype, device=x.device)
+        self.core.attend(lat, q, cache, ctx, group, k=pool, v=pool)
+        out = torch.empty((T, H, self.vdim), dtype=x.dtype, device=x.device)
+        gate = p[:, self.g_off:self.g_off + H] if self.gated else None
+        ops.gemm_heads_nt(out, lat[:, :, :R], self.uv, gate)
+        return linear(out.view(T, H * self.vdim), self.o, blocked=self.o_blocked)

@@ -48,3 +48,47 @@ class RMSNorm(Part):
         x = as_tensor(x)
         y = ops.add_rmsnorm(x, residual, self.weight, self.eps)
         return y, (x if residual is None else residual)
+
+
+@register_part("norm", "dynamic_tanh")
+class DynamicTanh(Part):
+    """y = tanh(alpha * x) * weight + bias, elementwise: a norm without mean or variance
+    (Zhu, Chen, He, LeCun, Liu: "Transformers without Normalization"). ``alpha`` is a scalar
+    of the checkpoint. The arithmetic is float32; the result is in the engine's dtype.
+
+    With a residual: the sum is made in a float32 residual stream (``residual`` must be one;
+    it is updated in place), as the blocks that keep such a stream do in one kernel with the
+    norms around it (``params()`` hands them what they need)."""
+    kernel_libraries = ("stream",)
+
+    def __init__(self, size: int, weight_name: str = "weight", bias_name: str = "bias",
+                 alpha_name: str = "alpha"):
+        self.size = int(size)
+        self.names = (weight_name, bias_name, alpha_name)
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+        self.alpha = 1.0
+        self.dtype: Optional[torch.dtype] = None
+
+    def param_sources(self) -> List[ParamSource]:
+        w, b, a = self.names
+        return [ParamSource(w, (self.size,), "vector"),
+                ParamSource(b, (self.size,), "vector", init=("normal", 0.0, 0.1)),
+                ParamSource(a, (), "vector", init=("uniform", 0.4, 1.2))]
+
+    def load(self, tensors, dtype, device) -> None:
+        w, b, a = self.names
+        self.weight = place(tensors[w], "vector", dtype, device)
+        self.bias = place(tensors[b], "vector", dtype, device)
+        self.alpha = float(tensors[a].float().item())        # (a host tensor of the checkpoint)
+        self.dtype = dtype
+
+    def params(self):
+        return (self.weight, self.bias, self.alpha)
+
+    def forward(self, x, residual: Optional[torch.Tensor]):
+        x = as_tensor(x)
+        if residual is None:
+            return ops.dyt(x, self.weight, self.bias, self.alpha, self.dtype), x
+        y, _ = ops.stream_add_dyt(residual, x, None, self.params(), self.dtype)
+        return y, residual
