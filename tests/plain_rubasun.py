@@ -76,10 +76,16 @@ def clamped_expert(h, W, prefix, limit):
     return (g * torch.sigmoid(1.702 * g) * (u + 1)) @ W[prefix + ".down"].T
 
 
-def moe_ff(h, W, prefix, mlp):
+def moe_ff(h, W, prefix, mlp, margins_out=None):
+    """``margins_out``: a list that receives, per token, by how much the logit of its last
+    chosen expert exceeds that of the best expert left out (inf when all are chosen)."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
-    s = torch.sigmoid(h @ W[prefix + ".router"].T)                  # [T, E]
+    z = h @ W[prefix + ".router"].T                                 # [T, E]
+    s = torch.sigmoid(z)
     val, idx = torch.topk(s, top, dim=-1)
+    if margins_out is not None:
+        zs = z.sort(-1, descending=True).values
+        margins_out.append(zs[:, top - 1] - zs[:, top] if top < E else torch.full_like(zs[:, 0], float("inf")))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for k in range(top):
@@ -102,9 +108,9 @@ def norm_of(x, W, name):
     return dyt(x, W[name], W[name + ".b"], W[name + ".alpha"])
 
 
-def forward(cfg, weights, tokens, dtype=torch.float32, round_to=None, layers_out=None):
+def forward(cfg, weights, tokens, dtype=torch.float32, round_to=None, layers_out=None, margins_out=None):
     """Logits [T, vocab] of one whole sequence. ``layers_out``: a list that receives the
-    residual stream after every layer."""
+    residual stream after every layer; ``margins_out``: see moe_ff (one entry a routed layer)."""
     W = {}
     for k, t in weights.items():
         if t.dtype in (torch.int32, torch.int64):
@@ -131,7 +137,7 @@ def forward(cfg, weights, tokens, dtype=torch.float32, round_to=None, layers_out
         mlp = layer.get("mlp")
         if mlp is not None:
             h = norm_of(x, W, name + ".norm2")
-            y = dense_ff(h, W, name + ".mlp") if mlp["kind"] == "dense" else moe_ff(h, W, name + ".mlp", mlp)
+            y = dense_ff(h, W, name + ".mlp") if mlp["kind"] == "dense" else moe_ff(h, W, name + ".mlp", mlp, margins_out)
             x = x + norm_of(y, W, name + ".norm2b")
         if cfg.get("token_side"):
             x = token_side(x, tokens, W, name, i, cfg["token_side"]["dim"], eps)
