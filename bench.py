@@ -202,6 +202,121 @@ def like_reference(args, cfg, short):
     return 0
 
 
+def rubasun_shape(width, layers, heads, dim, rot_dim, vdim, kv_rank, dense_ff, experts, top, expert_ff,
+                  shared_ff, side_dim, vocab):
+    """A Rubasun config.json of a real model's layer sizes: the first layer dense, the others
+    routed; every third layer keeps a latent cache of its own and the two behind it read it."""
+    def mixer(kv_from):
+        m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank,
+             "scale": (dim + rot_dim) ** -0.5, "rot": {"base": 10000.0, "dims": rot_dim}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return m
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff, "limit": 7.0},
+           "shared": {"ff": shared_ff, "limit": 7.0}}
+    out = []
+    for i in range(layers):
+        owner = i - i % 3
+        out.append({"type": "latent_attention", "mixer": mixer(None if owner == i else owner),
+                    "mlp": {"kind": "dense", "ff": dense_ff} if i == 0 else moe})
+    return {"architecture": "Rubasun", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "token_side": {"dim": side_dim}, "layers": out, "initializer_range": 0.02}
+
+
+# name -> (Rubasun sizes, the Llama shape of equal width, depth and feed-forward width a token)
+RUBASUN_SIZES = {
+    "2048": (dict(width=2048, layers=8, heads=16, dim=64, rot_dim=32, vdim=64, kv_rank=96, dense_ff=8192,
+                  experts=16, top=2, expert_ff=2048, shared_ff=4096, side_dim=64, vocab=32000),
+             dict(num_hidden_layers=8, hidden_size=2048, num_attention_heads=32, num_key_value_heads=8,
+                  head_dim=64, intermediate_size=8192, vocab_size=32000, tie_word_embeddings=False)),
+    "4096": (dict(width=4096, layers=4, heads=32, dim=64, rot_dim=32, vdim=64, kv_rank=96, dense_ff=14336,
+                  experts=32, top=4, expert_ff=2048, shared_ff=6144, side_dim=128, vocab=32000),
+             dict(num_hidden_layers=4, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                  head_dim=128, intermediate_size=14336, vocab_size=32000, tie_word_embeddings=False)),
+}
+
+
+def engine_rates(cfg, dtype, S, batch, steps, warmup):
+    """Prefill of one S-token prompt (one step) and decode steps of ``batch`` requests behind
+    S-token prompts, through the whole engine, for any architecture."""
+    import torch
+    from pytriton_llama_amd.config import EngineConfig
+    from pytriton_llama_amd.engine import Engine, SamplingParams
+    page = 16
+    room = S + steps + warmup + 16
+    ec = EngineConfig(dtype=dtype, page_size=page, num_pages=-(-room // page) * batch + 8, max_num_seqs=batch,
+                      max_num_batched_tokens=max(S, 2048), max_model_len=room, seed=0)
+    engine = Engine(cfg, ec, random_seed=0)
+    vocab = engine.model.vocab_size
+    g = torch.Generator().manual_seed(4321)
+    prompt = lambda: torch.randint(0, vocab, (S,), generator=g).tolist()
+    times = []
+    for _ in range(6):
+        rid = engine.add_request(prompt(), SamplingParams(temperature=0.0, max_new_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        while engine.has_work:
+            engine.step()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t)
+        engine.requests.pop(rid, None)
+    pre = min(times[1:])
+    ids = [engine.add_request(prompt(), SamplingParams(temperature=0.0, max_new_tokens=steps + warmup,
+                                                       ignore_eos=True)) for _ in range(batch)]
+    while any(engine.requests[i].num_computed < S for i in ids):
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    for i in ids:
+        engine.requests[i].params.max_new_tokens = len(engine.requests[i].output) + steps
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    made = 0
+    for _ in range(steps):
+        made += len(engine.step())
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t
+    assert made == batch * steps and not engine.has_work, (made, batch, steps)
+    params = sum(t.numel() for t in _tensors_of(engine.model))
+    del engine
+    torch.cuda.empty_cache()
+    return {"prefill_ms": round(pre * 1e3, 3), "prefill_tokens_per_s": round(S / pre, 1),
+            "decode_ms_per_step": round(dt / steps * 1e3, 4), "decode_tokens_per_s": round(made / dt, 1),
+            "weights_held": params}
+
+
+def _tensors_of(model):
+    """The checkpoint's tensors as the model expects them (shapes only)."""
+    import torch
+    return [torch.empty(src.shape, device="meta") for _, src in model.expected_tensors().values()]
+
+
+def rubasun_beside_llama(args):
+    """Prefill and decode throughput of Rubasun at layer sizes of real models, beside the
+    Llama decoder of equal width, depth and feed-forward width a token, same engine, same
+    measurement. One JSON line."""
+    rows = {}
+    for name in [n for n in args.rubasun.split(",") if n]:
+        if name not in RUBASUN_SIZES:
+            print(f"--rubasun takes {sorted(RUBASUN_SIZES)}", file=sys.stderr)
+            return 2
+        r_sizes, l_shape = RUBASUN_SIZES[name]
+        llama = dict(LLAMA_1B)
+        llama.update(l_shape)
+        for label, cfg in (("rubasun", rubasun_shape(**r_sizes)), ("llama", llama)):
+            log(f"width {name}: {label}")
+            rows[f"{label}_{name}"] = engine_rates(cfg, args.dtype, args.prompt_len, args.batch, args.steps,
+                                                   args.warmup)
+            log(json.dumps(rows[f"{label}_{name}"]))
+    print(json.dumps({"metric": f"Rubasun beside Llama: prefill of {args.prompt_len} tokens and decode at batch "
+                                f"{args.batch} behind {args.prompt_len}-token prompts",
+                      "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                      "sizes": {n: {"rubasun": RUBASUN_SIZES[n][0], "llama": RUBASUN_SIZES[n][1]}
+                                for n in args.rubasun.split(",") if n}, "rows": rows}), flush=True)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -231,6 +346,10 @@ def main():
                     help="instead of the decode measurement: one generate() call of the Python entry point "
                          "for B short prompts, 256 new tokens, temperature 0.6, top_p 0.9, as the "
                          "reference's examples/benchmark.py measures")
+    ap.add_argument("--rubasun", default="", metavar="SIZES",
+                    help="instead of the decode measurement: the Rubasun design beside Llama at the named "
+                         "sizes (comma-separated, of: 2048, 4096): prefill of --prompt-len tokens and decode "
+                         "steps at --batch, both through the whole engine")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
@@ -255,6 +374,8 @@ def main():
     # requests whose prompt is in first go on decoding while the others' prompts are computed
     slack = max_batch * -(-S // (args.prefill_chunk or max(S, 2048))) + 8
     per_req_pages = -(-(S + max(W, K) + slack) // page)
+    if args.rubasun:
+        return rubasun_beside_llama(args)
     if args.mixed:
         return mixed_workload(args, cfg, short)
     if args.like_reference:
