@@ -23,7 +23,6 @@
 #include <math.h>
 
 #define MOE_TM 64
-#define MOE_SORT_LDS 8192      // pairs whose experts the sorting workgroup holds in LDS
 
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
 
@@ -106,11 +105,10 @@ __global__ void __launch_bounds__(1024)
 moe_sort_kernel(const int32_t* __restrict__ idx, int A, int E, int32_t* __restrict__ pos_of,
                 int32_t* __restrict__ sorted, int32_t* __restrict__ expert_end,
                 int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0, int max_tiles) {
-  extern __shared__ int32_t sh[];        // count [E], start [E], n_tiles [1], experts of the pairs [A]
+  extern __shared__ int32_t sh[];        // count [E], start [E], n_tiles [1]
   int32_t* count = sh;
   int32_t* start = sh + E;
   int32_t* n_tiles = sh + 2 * E;
-  int32_t* lidx = sh + 2 * E + 1;
   for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
   __syncthreads();
   for (int a = threadIdx.x; a < A; a += 1024) {
@@ -138,25 +136,8 @@ moe_sort_kernel(const int32_t* __restrict__ idx, int A, int E, int32_t* __restri
     tile_expert[i] = -1;
     tile_row0[i] = 0;
   }
-  // places inside an expert in the order of the pairs, so that the layout does not change from
-  // run to run: with the experts of all pairs in LDS, thread e walks them and hands expert e's
-  // places out in order (every thread reads the same word: a broadcast). More pairs than LDS
-  // holds: places by atomic counters (the order inside an expert then varies, the results
-  // of a row do not depend on its place).
-  if (A <= MOE_SORT_LDS) {
-    for (int a = threadIdx.x; a < A; a += 1024) lidx[a] = idx[a];
-    __syncthreads();
-    for (int e = threadIdx.x; e < E; e += 1024) {
-      int p = start[e];
-      const int end = expert_end[e];
-      for (int a = 0; a < A && p < end; ++a)
-        if (lidx[a] == e) {
-          sorted[p] = a;
-          pos_of[a] = p++;
-        }
-    }
-    return;
-  }
+  // places inside an expert by a counter in LDS: which pair gets which place varies from run
+  // to run, the results do not (a row's result does not depend on its place in a tile)
   for (int a = threadIdx.x; a < A; a += 1024) {
     const int e = idx[a];
     if (e < 0 || e >= E) continue;
@@ -173,7 +154,7 @@ extern "C" int ptl_moe_sort(const int32_t* idx, int A, int E, int32_t* pos_of, i
                             hipStream_t st) {
   if (A <= 0) return PTL_OK;
   if (E <= 0 || E > 8192 || max_tiles < ptl_moe_max_tiles(A, E)) return PTL_ERR_ARG;
-  moe_sort_kernel<<<1, 1024, (2 * E + 1 + (A <= MOE_SORT_LDS ? A : 0)) * sizeof(int32_t), st>>>(idx, A, E, pos_of, sorted, expert_end,
+  moe_sort_kernel<<<1, 1024, (2 * E + 1) * sizeof(int32_t), st>>>(idx, A, E, pos_of, sorted, expert_end,
                                                                   tile_expert, tile_row0, max_tiles);
   return ptl_launch_status();
 }
@@ -274,8 +255,12 @@ moe_gemm_kernel(T* __restrict__ out, long ldo, const T* __restrict__ x, long ldx
   }
 }
 
-// Matrix-core form for bfloat16 (K % 8 == 0, aligned rows): a wave owns 16 sorted rows x 64
-// columns, fragments straight from memory as in ptl_gemm_heads_nt.
+// Matrix-core forms for bfloat16 (K % 8 == 0, aligned rows).
+//
+// Few pairs (a decode step): fragments straight from memory, 64 result columns a workgroup. A
+// tile of at most 16 rows (nearly every tile of a decode step) is shared by the four waves
+// along K, 32 values in turn, so that four times as many loads of the expert's weights are under
+// way; their partial sums meet in LDS. Taller tiles: a wave owns 16 of the rows.
 template <bool GATE_UP>
 __global__ void __launch_bounds__(256)
 moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restrict__ x, long ldx,
@@ -283,13 +268,17 @@ moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restric
                      const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ expert_end,
                      const int32_t* __restrict__ sorted, const float* __restrict__ wgt, int top, int N, int K,
                      int act, float limit) {
+  constexpr int G = GATE_UP ? 2 : 1;
+  __shared__ float red[3][G * 4][4][64];
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int ln = lane & 15, lg = lane >> 4;
-  const int row0 = tile_row0[blockIdx.y] + 16 * wave;
+  const int tile_rows = min(MOE_TM, expert_end[e] - tile_row0[blockIdx.y]);
+  const bool split = tile_rows <= 16;
+  const int row0 = tile_row0[blockIdx.y] + (split ? 0 : 16 * wave);
   const int rows = min(16, expert_end[e] - row0);
-  if (rows <= 0) return;
+  if (rows <= 0) return;                 // (never in a split tile: its waves all stay)
   const int n0 = blockIdx.x * 64;
   const size_t wrows = GATE_UP ? 2 * (size_t)N : (size_t)N;
   w += (size_t)e * wrows * K;
@@ -305,27 +294,48 @@ moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restric
   const bf16_t* brow[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) brow[j] = w + (size_t)min(n0 + 16 * j + ln, N - 1) * K;
-  f32x4_t acc[GATE_UP ? 2 : 1][4];
+  f32x4_t acc[G][4];
 #pragma unroll
-  for (int g = 0; g < (GATE_UP ? 2 : 1); ++g)
+  for (int g = 0; g < G; ++g)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[g][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const uint4 zero = make_uint4(0, 0, 0, 0);
   const size_t up = (size_t)N * K;
-  for (int k0 = 0; k0 < K; k0 += 32) {
+  const int kstep = split ? 128 : 32;
+  for (int k0 = split ? 32 * wave : 0; k0 < K; k0 += kstep) {
     const int k = k0 + 8 * lg;
-    Frag8 a, b[GATE_UP ? 2 : 1][4];
+    Frag8 a, b[G][4];
     a.u = k < K ? *reinterpret_cast<const uint4*>(arow + k) : zero;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       b[0][j].u = k < K ? load_once(brow[j] + k) : zero;
-      if (GATE_UP) b[GATE_UP ? 1 : 0][j].u = k < K ? load_once(brow[j] + up + k) : zero;
+      if (GATE_UP) b[G - 1][j].u = k < K ? load_once(brow[j] + up + k) : zero;
     }
 #pragma unroll
-    for (int g = 0; g < (GATE_UP ? 2 : 1); ++g)
+    for (int g = 0; g < G; ++g)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         acc[g][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[g][j].v, a.v, acc[g][j], 0, 0, 0);
+  }
+  if (split) {
+    if (wave > 0) {
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) red[wave - 1][g * 4 + j][i][lane] = acc[g][j][i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int v = 0; v < 3; ++v)
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[g][j][i] += red[v][g * 4 + j][i][lane];
   }
   if (ln < rows) {
 #pragma unroll
@@ -336,13 +346,159 @@ moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restric
         if (n >= N) continue;
         float v;
         if (GATE_UP)
-          v = gated_act(act, acc[0][j][i] * f, acc[GATE_UP ? 1 : 0][j][i] * f, limit);
+          v = gated_act(act, acc[0][j][i] * f, acc[G - 1][j][i] * f, limit);
         else
           v = acc[0][j][i];
         out[(size_t)(row0 + ln) * ldo + n] = float_to_bf16(v);
       }
   }
 }
+
+// Many pairs (a prompt portion): tiles through LDS. A workgroup owns 64 sorted rows x 128 rows
+// of the expert's matrix (gate|up: 64 gate rows and the 64 up rows that belong to them, so that
+// the activation meets in one lane; down: 128 result columns); chunks of 64 along K, two buffers,
+// the next chunk on its way from memory while this one is multiplied; rows padded by 16 bytes
+// against bank conflicts. A wave owns 32 rows x 64 of the 128.
+#define TB_K 64
+#define TB_LD 72
+
+template <bool GATE_UP>
+__global__ void __launch_bounds__(256)
+moe_gemm_tiled_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restrict__ x, long ldx,
+                      const bf16_t* __restrict__ w, const int32_t* __restrict__ tile_expert,
+                      const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ expert_end,
+                      const int32_t* __restrict__ sorted, const float* __restrict__ wgt, int top, int N, int K,
+                      int act, float limit) {
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][64 * TB_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[2][128 * TB_LD];
+  __shared__ int32_t src_row[64];
+  __shared__ float row_w[64];
+  const int tid = threadIdx.x;
+  const int row0 = tile_row0[blockIdx.y];
+  const int rows = min(MOE_TM, expert_end[e] - row0);
+  if (tid < 64) {
+    int r = -1;
+    float f = 1.f;
+    if (tid < rows) {
+      if (GATE_UP) {
+        const int a = sorted[row0 + tid];
+        r = a / top;
+        if (wgt) f = wgt[a];
+      } else {
+        r = row0 + tid;
+      }
+    }
+    src_row[tid] = r;
+    row_w[tid] = f;
+  }
+  __syncthreads();
+  const int n0 = blockIdx.x * (GATE_UP ? 64 : 128);
+  const size_t wrows = GATE_UP ? 2 * (size_t)N : (size_t)N;
+  w += (size_t)e * wrows * K;
+  // what this thread brings of a chunk: 2 pieces of 16 bytes of x rows, 4 of weight rows
+  const int kc = (tid & 7) * 8;
+  const bf16_t* a_ptr[2];
+  const bf16_t* b_ptr[4];
+  int a_at[2], b_at[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = (tid + 256 * i) >> 3;
+    const int s = src_row[r];
+    a_ptr[i] = s >= 0 ? x + (size_t)s * ldx + kc : nullptr;
+    a_at[i] = r * TB_LD + kc;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = (tid + 256 * i) >> 3;
+    size_t grow;
+    bool ok;
+    if (GATE_UP) {
+      const int col = n0 + (r & 63);
+      ok = col < N;
+      grow = r < 64 ? (size_t)col : (size_t)N + col;
+    } else {
+      ok = n0 + r < N;
+      grow = (size_t)n0 + r;
+    }
+    b_ptr[i] = ok ? w + grow * K + kc : nullptr;
+    b_at[i] = r * TB_LD + kc;
+  }
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  uint4 ra[2], rb[4];
+  auto gload = [&](int k0) {
+    const bool in = k0 + kc < K;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) ra[i] = (a_ptr[i] && in) ? *reinterpret_cast<const uint4*>(a_ptr[i] + k0) : zero;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rb[i] = (b_ptr[i] && in) ? load_once(b_ptr[i] + k0) : zero;
+  };
+  auto sstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(&As[buf][a_at[i]]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(&Bs[buf][b_at[i]]) = rb[i];
+  };
+  const int wave = tid >> 6, lane = tid & 63;
+  const int ln = lane & 15, lg = lane >> 4;
+  const int rh = wave & 1, cg = wave >> 1;
+  int b_off[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    b_off[j] = GATE_UP ? (j >> 1) * 64 + cg * 32 + (j & 1) * 16 : cg * 64 + 16 * j;
+  f32x4_t acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  gload(0);
+  sstore(0);
+  __syncthreads();
+  const int chunks = (K + TB_K - 1) / TB_K;
+  for (int c = 0; c < chunks; ++c) {
+    const int buf = c & 1;
+    if (c + 1 < chunks) gload((c + 1) * TB_K);
+#pragma unroll
+    for (int ks = 0; ks < TB_K / 32; ++ks) {
+      Frag8 a[2], b[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i].u = *reinterpret_cast<const uint4*>(&As[buf][(rh * 32 + 16 * i + ln) * TB_LD + ks * 32 + 8 * lg]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        b[j].u = *reinterpret_cast<const uint4*>(&Bs[buf][(b_off[j] + ln) * TB_LD + ks * 32 + 8 * lg]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[j].v, a[i].v, acc[i][j], 0, 0, 0);
+    }
+    if (c + 1 < chunks) sstore(buf ^ 1);
+    __syncthreads();
+  }
+  // lane holds, of tile (i, j): row m = rh * 32 + 16 i + ln, weight rows b_off[j] + 4 lg + q
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = rh * 32 + 16 * i + ln;
+    if (m >= rows) continue;
+    const float f = row_w[m];
+    bf16_t* orow = out + (size_t)(row0 + m) * ldo;
+#pragma unroll
+    for (int j = 0; j < (GATE_UP ? 2 : 4); ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = GATE_UP ? n0 + cg * 32 + 16 * j + 4 * lg + q : n0 + cg * 64 + 16 * j + 4 * lg + q;
+        if (n >= N) continue;
+        const float v = GATE_UP ? gated_act(act, acc[i][j][q] * f, acc[i][GATE_UP ? j + 2 : j][q] * f, limit)
+                                : acc[i][j][q];
+        orow[n] = float_to_bf16(v);
+      }
+  }
+}
+
+// pairs from which on the tiles go through LDS (below: a decode step, tiles of a few rows)
+#define MOE_TILED_FROM 128
 
 static bool mfma_ok(const void* x, long ldx, const void* w, int K) {
   return K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x | (uintptr_t)w) % 16 == 0;
@@ -353,7 +509,7 @@ static bool mfma_ok(const void* x, long ldx, const void* w, int K) {
 extern "C" int ptl_moe_gate_up(void* out, long ldo, const void* x, long ldx, const void* w,
                                const int32_t* tile_expert, const int32_t* tile_row0,
                                const int32_t* expert_end, const int32_t* sorted, const float* wgt,
-                               int max_tiles, int top, int I, int K, int act, float limit, int dtype,
+                               int max_tiles, int pairs, int top, int I, int K, int act, float limit, int dtype,
                                hipStream_t st) {
   if (max_tiles <= 0) return PTL_OK;
   if (I <= 0 || K <= 0 || top <= 0 || max_tiles > 65535) return PTL_ERR_ARG;
@@ -362,6 +518,10 @@ extern "C" int ptl_moe_gate_up(void* out, long ldo, const void* x, long ldx, con
     moe_gemm_kernel<float, true><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
                                                        tile_expert, tile_row0, expert_end, sorted, wgt, top, I,
                                                        K, act, limit);
+  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM)
+    moe_gemm_tiled_kernel<true><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                      (const bf16_t*)w, tile_expert, tile_row0, expert_end,
+                                                      sorted, wgt, top, I, K, act, limit);
   else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
     moe_gemm_mfma_kernel<true><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                      (const bf16_t*)w, tile_expert, tile_row0, expert_end,
@@ -378,7 +538,7 @@ extern "C" int ptl_moe_gate_up(void* out, long ldo, const void* x, long ldx, con
 // out [A, N] (sorted order) = x [A, K] (sorted order) Wd_e^T; w [E, N, K]
 extern "C" int ptl_moe_down(void* out, long ldo, const void* x, long ldx, const void* w,
                             const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* expert_end,
-                            int max_tiles, int N, int K, int dtype, hipStream_t st) {
+                            int max_tiles, int pairs, int N, int K, int dtype, hipStream_t st) {
   if (max_tiles <= 0) return PTL_OK;
   if (N <= 0 || K <= 0 || max_tiles > 65535) return PTL_ERR_ARG;
   dim3 grid((N + 63) / 64, max_tiles);
@@ -386,7 +546,12 @@ extern "C" int ptl_moe_down(void* out, long ldo, const void* x, long ldx, const 
     moe_gemm_kernel<float, false><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
                                                         tile_expert, tile_row0, expert_end, nullptr, nullptr, 1,
                                                         N, K, 0, 0.f);
-  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
+  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM) {
+    dim3 wide((N + 127) / 128, max_tiles);
+    moe_gemm_tiled_kernel<false><<<wide, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                       (const bf16_t*)w, tile_expert, tile_row0, expert_end,
+                                                       nullptr, nullptr, 1, N, K, 0, 0.f);
+  } else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
     moe_gemm_mfma_kernel<false><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                       (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                       nullptr, nullptr, 1, N, K, 0, 0.f);

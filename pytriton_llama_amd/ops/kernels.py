@@ -1179,11 +1179,11 @@ def moe_experts(x: torch.Tensor, r: Routing, gate_up: torch.Tensor, down: torch.
     mid = torch.empty((A, I), dtype=x.dtype, device=x.device)
     _check(lib.ptl_moe_gate_up(_ptr(mid), ctypes.c_long(I), _ptr(x), ctypes.c_long(x.stride(0)), _ptr(gate_up),
                                _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), _ptr(r.sorted),
-                               _ptr(r.wgt) if weight_on_input else None, r.max_tiles, r.top, I, K, int(act),
+                               _ptr(r.wgt) if weight_on_input else None, r.max_tiles, A, r.top, I, K, int(act),
                                ctypes.c_float(limit), code, _stream()), "moe_gate_up")
     rows = torch.empty((A, N), dtype=x.dtype, device=x.device)
     _check(lib.ptl_moe_down(_ptr(rows), ctypes.c_long(N), _ptr(mid), ctypes.c_long(I), _ptr(down),
-                            _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), r.max_tiles, N, I,
+                            _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), r.max_tiles, A, N, I,
                             code, _stream()), "moe_down")
     y = torch.empty((T, N), dtype=torch.float32, device=x.device)
     _check(lib.ptl_moe_combine(_ptr(y), _ptr(rows), ctypes.c_long(N), _ptr(r.pos_of),

@@ -114,7 +114,8 @@ def test_per_head_products(gpu_device, dtype, K, N):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
-@pytest.mark.parametrize("T,E,top,I", [(1, 4, 1, 24), (7, 5, 2, 40), (150, 6, 3, 72), (300, 70, 4, 16)])
+@pytest.mark.parametrize("T,E,top,I", [(1, 4, 1, 24), (7, 5, 2, 40), (40, 2, 1, 24), (150, 6, 3, 72), (300, 70, 4, 16),
+                                        (260, 3, 2, 200)])
 def test_routed_experts(gpu_device, dtype, T, E, top, I):
     """Routing, grouping and the experts' products against a loop over tokens; the weight
     scales the expert's input (with the clamp in the activation that is not the same as
