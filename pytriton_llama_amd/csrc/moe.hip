@@ -356,11 +356,15 @@ moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restric
 
 // Many pairs (a prompt portion): tiles through LDS. A workgroup owns 64 sorted rows x 128 rows
 // of the expert's matrix (gate|up: 64 gate rows and the 64 up rows that belong to them, so that
-// the activation meets in one lane; down: 128 result columns); chunks of 64 along K, two buffers,
-// the next chunk on its way from memory while this one is multiplied; rows padded by 16 bytes
-// against bank conflicts. A wave owns 32 rows x 64 of the 128.
+// the activation meets in one lane; down: 128 result columns); a wave owns 32 rows x 64 of the
+// 128. Chunks of 64 along K go from global memory straight into LDS (global_load_lds_dwordx4:
+// every lane names its own 16 bytes, a wave's 64 pieces land side by side, no register carries
+// them), two buffers, the next chunk in flight while this one is multiplied. Rows lie unpadded
+// (128 bytes); the 16-byte pieces of a row are permuted by the row number (piece c of row r lies
+// at c ^ ((r >> 1) & 7)), which keeps the fragment reads free of bank conflicts. Rows past the
+// tile's end read some valid row (their results are never stored). Needs K % 64 == 0.
 #define TB_K 64
-#define TB_LD 72
+#define TB_BROWS 128
 
 template <bool GATE_UP>
 __global__ void __launch_bounds__(256)
@@ -371,113 +375,114 @@ moe_gemm_tiled_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restri
                       int act, float limit) {
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
-  __shared__ __attribute__((aligned(16))) bf16_t As[2][64 * TB_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Bs[2][128 * TB_LD];
+  __shared__ __attribute__((aligned(1024))) bf16_t As0[64 * TB_K];
+  __shared__ __attribute__((aligned(1024))) bf16_t As1[64 * TB_K];
+  __shared__ __attribute__((aligned(1024))) bf16_t Bs0[TB_BROWS * TB_K];
+  __shared__ __attribute__((aligned(1024))) bf16_t Bs1[TB_BROWS * TB_K];
   __shared__ int32_t src_row[64];
   __shared__ float row_w[64];
   const int tid = threadIdx.x;
   const int row0 = tile_row0[blockIdx.y];
   const int rows = min(MOE_TM, expert_end[e] - row0);
   if (tid < 64) {
-    int r = -1;
+    const int t = min(tid, rows - 1);
+    int r;
     float f = 1.f;
-    if (tid < rows) {
-      if (GATE_UP) {
-        const int a = sorted[row0 + tid];
-        r = a / top;
-        if (wgt) f = wgt[a];
-      } else {
-        r = row0 + tid;
-      }
+    if (GATE_UP) {
+      const int a = sorted[row0 + t];
+      r = a / top;
+      if (wgt) f = wgt[a];
+    } else {
+      r = row0 + t;
     }
     src_row[tid] = r;
     row_w[tid] = f;
   }
   __syncthreads();
-  const int n0 = blockIdx.x * (GATE_UP ? 64 : 128);
+  const int n0 = blockIdx.x * (GATE_UP ? TB_BROWS / 2 : TB_BROWS);
   const size_t wrows = GATE_UP ? 2 * (size_t)N : (size_t)N;
   w += (size_t)e * wrows * K;
-  // what this thread brings of a chunk: 2 pieces of 16 bytes of x rows, 4 of weight rows
-  const int kc = (tid & 7) * 8;
-  const bf16_t* a_ptr[2];
-  const bf16_t* b_ptr[4];
-  int a_at[2], b_at[4];
+  const int wave = tid >> 6, lane = tid & 63;
+  // the pieces this lane names: slot s = 64 (instruction) + lane holds row s / 8, piece (s % 8) ^ swz
+  const bf16_t* a_src[2];
+  const bf16_t* b_src[4];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    const int r = (tid + 256 * i) >> 3;
-    const int s = src_row[r];
-    a_ptr[i] = s >= 0 ? x + (size_t)s * ldx + kc : nullptr;
-    a_at[i] = r * TB_LD + kc;
+    const int slot = 64 * (wave * 2 + i) + lane;
+    const int r = slot >> 3, c = (slot & 7) ^ ((r >> 1) & 7);
+    a_src[i] = x + (size_t)src_row[r] * ldx + 8 * c;
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int r = (tid + 256 * i) >> 3;
+    const int slot = 64 * (wave * 4 + i) + lane;
+    const int r = slot >> 3, c = (slot & 7) ^ ((r >> 1) & 7);
     size_t grow;
-    bool ok;
     if (GATE_UP) {
-      const int col = n0 + (r & 63);
-      ok = col < N;
+      const int col = min(n0 + (r & 63), N - 1);
       grow = r < 64 ? (size_t)col : (size_t)N + col;
     } else {
-      ok = n0 + r < N;
-      grow = (size_t)n0 + r;
+      grow = (size_t)min(n0 + r, N - 1);
     }
-    b_ptr[i] = ok ? w + grow * K + kc : nullptr;
-    b_at[i] = r * TB_LD + kc;
+    b_src[i] = w + grow * K + 8 * c;
   }
-  const uint4 zero = make_uint4(0, 0, 0, 0);
-  uint4 ra[2], rb[4];
-  auto gload = [&](int k0) {
-    const bool in = k0 + kc < K;
+  auto fetch = [&](int k0, bf16_t* Ab, bf16_t* Bb) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) ra[i] = (a_ptr[i] && in) ? *reinterpret_cast<const uint4*>(a_ptr[i] + k0) : zero;
+    for (int i = 0; i < 2; ++i)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[i] + k0),
+                                       (__attribute__((address_space(3))) void*)(Ab + 512 * (wave * 2 + i)), 16, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) rb[i] = (b_ptr[i] && in) ? load_once(b_ptr[i] + k0) : zero;
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[i] + k0),
+                                       (__attribute__((address_space(3))) void*)(Bb + 512 * (wave * 4 + i)), 16, 0, 0);
   };
-  auto sstore = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(&As[buf][a_at[i]]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(&Bs[buf][b_at[i]]) = rb[i];
-  };
-  const int wave = tid >> 6, lane = tid & 63;
   const int ln = lane & 15, lg = lane >> 4;
   const int rh = wave & 1, cg = wave >> 1;
-  int b_off[4];
+  // where this lane reads its fragments: row * 64 elements, piece (4 ks + lg) ^ swz(row)
+  int a_row[2], b_row[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) a_row[i] = rh * 32 + 16 * i + ln;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
-    b_off[j] = GATE_UP ? (j >> 1) * 64 + cg * 32 + (j & 1) * 16 : cg * 64 + 16 * j;
+    b_row[j] = (GATE_UP ? (j >> 1) * 64 + cg * 32 + (j & 1) * 16 : cg * 64 + 16 * j) + ln;
   f32x4_t acc[2][4];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  gload(0);
-  sstore(0);
-  __syncthreads();
-  const int chunks = (K + TB_K - 1) / TB_K;
-  for (int c = 0; c < chunks; ++c) {
-    const int buf = c & 1;
-    if (c + 1 < chunks) gload((c + 1) * TB_K);
+  auto mult = [&](const bf16_t* Ab, const bf16_t* Bb) {
 #pragma unroll
-    for (int ks = 0; ks < TB_K / 32; ++ks) {
+    for (int ks = 0; ks < 2; ++ks) {
       Frag8 a[2], b[4];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-        a[i].u = *reinterpret_cast<const uint4*>(&As[buf][(rh * 32 + 16 * i + ln) * TB_LD + ks * 32 + 8 * lg]);
+        a[i].u = *reinterpret_cast<const uint4*>(Ab + a_row[i] * TB_K + 8 * ((4 * ks + lg) ^ ((a_row[i] >> 1) & 7)));
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        b[j].u = *reinterpret_cast<const uint4*>(&Bs[buf][(b_off[j] + ln) * TB_LD + ks * 32 + 8 * lg]);
+        b[j].u = *reinterpret_cast<const uint4*>(Bb + b_row[j] * TB_K + 8 * ((4 * ks + lg) ^ ((b_row[j] >> 1) & 7)));
+      __builtin_amdgcn_sched_barrier(0);       // all reads of the stage first, then its products
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[j].v, a[i].v, acc[i][j], 0, 0, 0);
     }
-    if (c + 1 < chunks) sstore(buf ^ 1);
+  };
+  const int chunks = K / TB_K;
+  fetch(0, As0, Bs0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): this wave's loads into LDS have landed
+  __syncthreads();
+  for (int c = 0; c < chunks; c += 2) {
+    if (c + 1 < chunks) fetch((c + 1) * TB_K, As1, Bs1);
+    mult(As0, Bs0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (c + 1 >= chunks) break;
+    if (c + 2 < chunks) fetch((c + 2) * TB_K, As0, Bs0);
+    mult(As1, Bs1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
   }
-  // lane holds, of tile (i, j): row m = rh * 32 + 16 i + ln, weight rows b_off[j] + 4 lg + q
+  // lane holds, of tile (i, j): row m = rh * 32 + 16 i + ln, weight rows (b_row[j] - ln) + 4 lg + q
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int m = rh * 32 + 16 * i + ln;
@@ -518,10 +523,12 @@ extern "C" int ptl_moe_gate_up(void* out, long ldo, const void* x, long ldx, con
     moe_gemm_kernel<float, true><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
                                                        tile_expert, tile_row0, expert_end, sorted, wgt, top, I,
                                                        K, act, limit);
-  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM)
-    moe_gemm_tiled_kernel<true><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM && K % TB_K == 0) {
+    dim3 wide((I + TB_BROWS / 2 - 1) / (TB_BROWS / 2), max_tiles);
+    moe_gemm_tiled_kernel<true><<<wide, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                       (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                       sorted, wgt, top, I, K, act, limit);
+  }
   else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
     moe_gemm_mfma_kernel<true><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                      (const bf16_t*)w, tile_expert, tile_row0, expert_end,
@@ -546,8 +553,8 @@ extern "C" int ptl_moe_down(void* out, long ldo, const void* x, long ldx, const 
     moe_gemm_kernel<float, false><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
                                                         tile_expert, tile_row0, expert_end, nullptr, nullptr, 1,
                                                         N, K, 0, 0.f);
-  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM) {
-    dim3 wide((N + 127) / 128, max_tiles);
+  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM && K % TB_K == 0) {
+    dim3 wide((N + TB_BROWS - 1) / TB_BROWS, max_tiles);
     moe_gemm_tiled_kernel<false><<<wide, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                        (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                        nullptr, nullptr, 1, N, K, 0, 0.f);

@@ -114,14 +114,15 @@ def test_per_head_products(gpu_device, dtype, K, N):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
-@pytest.mark.parametrize("T,E,top,I", [(1, 4, 1, 24), (7, 5, 2, 40), (40, 2, 1, 24), (150, 6, 3, 72), (300, 70, 4, 16),
-                                        (260, 3, 2, 200)])
-def test_routed_experts(gpu_device, dtype, T, E, top, I):
+@pytest.mark.parametrize("T,E,top,I,W", [(1, 4, 1, 24, 48), (7, 5, 2, 40, 48), (40, 2, 1, 24, 48),
+                                          (150, 6, 3, 72, 48), (300, 70, 4, 16, 48), (260, 3, 2, 200, 48),
+                                          (200, 4, 2, 192, 128), (333, 9, 3, 64, 64)])
+def test_routed_experts(gpu_device, dtype, T, E, top, I, W):
     """Routing, grouping and the experts' products against a loop over tokens; the weight
     scales the expert's input (with the clamp in the activation that is not the same as
     scaling its output)."""
     from pytriton_llama_amd.parts import GatedMLP, RoutedExperts
-    W, limit = 48, 0.8
+    limit = 0.8
     tensors = {"router": rnd(E, W, seed=1, std=0.5), "shared.sg": rnd(1, W, seed=2, std=0.3)}
     for n, s in (("gate", 3), ("up", 4)):
         tensors["shared." + n] = rnd(32, W, seed=s, std=0.3)
