@@ -304,6 +304,8 @@ def rubasun_beside_llama(args):
         llama = dict(LLAMA_1B)
         llama.update(l_shape)
         for label, cfg in (("rubasun", rubasun_shape(**r_sizes)), ("llama", llama)):
+            if label not in args.rubasun_models.split(","):
+                continue
             log(f"width {name}: {label}")
             rows[f"{label}_{name}"] = engine_rates(cfg, args.dtype, args.prompt_len, args.batch, args.steps,
                                                    args.warmup)
@@ -350,6 +352,8 @@ def main():
                     help="instead of the decode measurement: the Rubasun design beside Llama at the named "
                          "sizes (comma-separated, of: 2048, 4096): prefill of --prompt-len tokens and decode "
                          "steps at --batch, both through the whole engine")
+    ap.add_argument("--rubasun-models", default="rubasun,llama",
+                    help="with --rubasun: which of the two models to run (for profiles of one of them)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")

@@ -593,6 +593,37 @@ moe_combine_kernel(float* __restrict__ y, const T* __restrict__ rows, long ldr, 
   y[t * N + n] = s;
 }
 
+// bfloat16 rows with N a multiple of 8 and aligned row starts: 8 columns a thread
+__global__ void __launch_bounds__(256)
+moe_combine_bf16_vec_kernel(float* __restrict__ y, const bf16_t* __restrict__ rows, long ldr,
+                            const int32_t* __restrict__ pos_of, const float* __restrict__ wgt, int top,
+                            const bf16_t* __restrict__ shared, const float* __restrict__ gate, int ldg, int N8) {
+  const size_t t = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= N8) return;
+  float s[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s[j] = 0.f;
+  union V { uint4 u; bf16_t e[8]; };
+  for (int k = 0; k < top; ++k) {
+    V v;
+    v.u = load_once(rows + (size_t)pos_of[t * top + k] * ldr + 8 * c);
+    const float f = wgt ? wgt[t * top + k] : 1.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s[j] += bf16_to_float(v.e[j]) * f;
+  }
+  if (shared) {
+    V v;
+    v.u = load_once(shared + (t * N8 + c) * 8);
+    const float f = gate ? gate[t * ldg] : 1.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s[j] += bf16_to_float(v.e[j]) * f;
+  }
+  float4* dst = reinterpret_cast<float4*>(y + (t * N8 + c) * 8);
+  dst[0] = make_float4(s[0], s[1], s[2], s[3]);
+  dst[1] = make_float4(s[4], s[5], s[6], s[7]);
+}
+
 extern "C" int ptl_moe_combine(float* y, const void* rows, long ldr, const int32_t* pos_of, const float* wgt,
                                int top, const void* shared, const float* gate, int ldg, int T_, int N, int dtype,
                                hipStream_t st) {
@@ -602,6 +633,14 @@ extern "C" int ptl_moe_combine(float* y, const void* rows, long ldr, const int32
     const int nt = T_ - t0 < 65535 ? T_ - t0 : 65535;
     dim3 grid((N + 255) / 256, nt);
     const size_t o = (size_t)t0;
+    if (dtype == PTL_DTYPE_BF16 && N % 8 == 0 && ldr % 8 == 0 &&
+        ((uintptr_t)rows | (uintptr_t)shared) % 16 == 0 && (uintptr_t)y % 16 == 0) {
+      dim3 vgrid((N / 8 + 255) / 256, nt);
+      moe_combine_bf16_vec_kernel<<<vgrid, 256, 0, st>>>(
+          y + o * N, (const bf16_t*)rows, ldr, pos_of + o * top, wgt ? wgt + o * top : nullptr, top,
+          shared ? (const bf16_t*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg, N / 8);
+      continue;
+    }
     if (dtype == PTL_DTYPE_F32)
       moe_combine_kernel<float><<<grid, 256, 0, st>>>(
           y + o * N, (const float*)rows, ldr, pos_of + o * top, wgt ? wgt + o * top : nullptr, top,
@@ -628,11 +667,32 @@ gated_act_kernel(T* __restrict__ out, const T* __restrict__ gu, int I, size_t to
   }
 }
 
+// bfloat16 rows with I a multiple of 8: 16-byte loads (marked as read once) and stores
+__global__ void __launch_bounds__(256)
+gated_act_bf16_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ gu, int I8, int act, float limit) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= I8) return;
+  const size_t t = blockIdx.y;
+  const bf16_t* row = gu + (t * 2 * I8 + c) * 8;
+  union { uint4 u; bf16_t e[8]; } g, u, o;
+  g.u = load_once(row);
+  u.u = load_once(row + (size_t)I8 * 8);
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    o.e[j] = float_to_bf16(gated_act(act, bf16_to_float(g.e[j]), bf16_to_float(u.e[j]), limit));
+  *reinterpret_cast<uint4*>(out + (t * I8 + c) * 8) = o.u;
+}
+
 // out [T, I] = act(gu[:, :I], gu[:, I:]) for a dense gate|up product [T, 2 I]
 extern "C" int ptl_gated_act(void* out, const void* gate_up, int T_, int I, int act, float limit, int dtype,
                              hipStream_t st) {
   if (T_ <= 0) return PTL_OK;
   if (I <= 0) return PTL_ERR_ARG;
+  if (dtype == PTL_DTYPE_BF16 && I % 8 == 0 && T_ <= 65535 && ((uintptr_t)out | (uintptr_t)gate_up) % 16 == 0) {
+    dim3 grid((I / 8 + 255) / 256, T_);
+    gated_act_bf16_vec_kernel<<<grid, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)gate_up, I / 8, act, limit);
+    return ptl_launch_status();
+  }
   const size_t total = (size_t)T_ * I;
   size_t blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;
