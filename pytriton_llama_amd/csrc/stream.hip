@@ -1,7 +1,7 @@
 // A residual stream that is kept in float32 whatever the engine's dtype, and the norms that read
 // and feed it:
 //
-//   Dynamic Tanh          y = tanh(alpha * x) * w + b            (no mean, no variance)
+//   Dynamic Tanh          y = tanh(alpha * x) * w + b            (elementwise, nothing of the row)
 //   RMS norm              y = x * rsqrt(mean(x^2) + eps) * w
 //
 // ptl_stream_add_dyt: stream += post(y) and out = pre(stream) in one pass over the rows: the norm

@@ -52,7 +52,7 @@ class RMSNorm(Part):
 
 @register_part("norm", "dynamic_tanh")
 class DynamicTanh(Part):
-    """y = tanh(alpha * x) * weight + bias, elementwise: a norm without mean or variance
+    """y = tanh(alpha * x) * weight + bias, elementwise: a norm that takes no statistics of its row
     (Zhu, Chen, He, LeCun, Liu: "Transformers without Normalization"). ``alpha`` is a scalar
     of the checkpoint. The arithmetic is float32; the result is in the engine's dtype.
 

@@ -75,8 +75,23 @@ def _r4():
     ])
 
 
+def _r5():
+    """Two cache shapes in one model (two page pools, two block tables a request), heads and
+    sizes that change from layer to layer, a borrowed cache behind each."""
+    a = dict(heads=2, dim=8, rot_dim=16, vdim=8, kv_rank=16, scale=0.3, base=1000.0)
+    b = dict(heads=6, dim=16, rot_dim=8, vdim=16, kv_rank=56, scale=0.2, base=20000.0, rot_dims=4)
+    a2 = dict(a, heads=4, dim=4, vdim=20)
+    return model(90, 80, 4.0, 1e-5, 3, [
+        layer(mixer(**a), dense(40)),
+        layer(mixer(**b), moe(6, 2, 16, 2.0, 8, 2.0)),
+        layer(mixer(**a2, kv_from=0), moe(6, 1, 16, 2.0)),
+        layer(mixer(**b, kv_from=1), dense(64)),
+    ])
+
+
 # name -> (config, weight std, page size)
-RUBASUN = {"R1": (_r1(), 0.12, 16), "R2": (_r2(), 0.10, 4), "R3": (_r3(), 0.10, 8), "R4": (_r4(), 0.15, 16)}
+RUBASUN = {"R1": (_r1(), 0.12, 16), "R2": (_r2(), 0.10, 4), "R3": (_r3(), 0.10, 8), "R4": (_r4(), 0.15, 16),
+           "R5": (_r5(), 0.15, 8)}
 
 
 def rubasun(name):
