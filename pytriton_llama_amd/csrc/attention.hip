@@ -17,14 +17,16 @@
 // of every window may be gone (table entry < 0) and are never touched.
 //
 // ptl_attention_generic: vector-FMA kernel, float32 math, storage type T
-// (float32 or bfloat16), any page size, any D up to 256.
+// (float32 or bfloat16), any page size, any D up to 640 (beyond 256 with more LDS than a
+// kernel gets unasked: the launcher asks for it).
 #include "common.h"
 #include "mfma.h"
 #include <math.h>
 
 #define BM 16
 
-template <typename T, int BN>
+// NJ: head-size columns a thread accumulates, 16 apart (16: head sizes up to 256; 40: up to 640)
+template <typename T, int BN, int NJ = 16>
 __global__ void __launch_bounds__(256)
 attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q, long q_stride,
                     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -66,9 +68,9 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
   const int nd = (D + 15) >> 4;
 
   float m_run = -INFINITY, l_run = 0.f;
-  float acc[16];
+  float acc[NJ];
 #pragma unroll
-  for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+  for (int j = 0; j < NJ; ++j) acc[j] = 0.f;
 
   for (int k0 = k_begin; k0 < k_end; k0 += BN) {
     __syncthreads();
@@ -120,7 +122,7 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
     l_run = l_run * alpha + psum;
     m_run = m_new;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) acc[j] *= alpha;
+    for (int j = 0; j < NJ; ++j) acc[j] *= alpha;
     __syncthreads();
 
     const int n_lim = min(BN, k_end - k0);
@@ -128,7 +130,7 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
       const float p = Ss[tm * BN + n];
       const float* vr = Vs + n * D + tc;
 #pragma unroll
-      for (int j = 0; j < 16; ++j)
+      for (int j = 0; j < NJ; ++j)
         if (j < nd && tc + 16 * j < D) acc[j] = fmaf(p, vr[16 * j], acc[j]);
     }
   }
@@ -137,12 +139,12 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
     T* o = out + (size_t)(qs + qoff + tm) * out_stride + head * D + tc;
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
+    for (int j = 0; j < NJ; ++j)
       if (j < nd && tc + 16 * j < D) o[16 * j] = from_float<T>(acc[j] * inv);
   }
 }
 
-template <typename T, int BN>
+template <typename T, int BN, int NJ = 16>
 static int launch_generic(void* out, long out_stride, const void* q, long q_stride,
                           const void* k_cache, const void* v_cache, const int32_t* q_start,
                           const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
@@ -150,8 +152,20 @@ static int launch_generic(void* out, long out_stride, const void* q, long q_stri
                           int Hq, int Hkv, int D, int page_size, int window, float scale,
                           hipStream_t stream) {
   const size_t lds = (size_t)(BM * D + BN * (D + 1) + BN * D + BM * BN) * sizeof(float);
+  if (lds > 64 * 1024) {
+    // more dynamic LDS than a kernel may ask for without saying so beforehand (wide heads only)
+    static size_t allowed = 0;
+    if (lds > allowed) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_generic_kernel<T, BN, NJ>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return PTL_ERR_ARG;
+      }
+      allowed = lds;
+    }
+  }
   dim3 grid(n_work, Hq);
-  attn_generic_kernel<T, BN><<<grid, 256, lds, stream>>>(
+  attn_generic_kernel<T, BN, NJ><<<grid, 256, lds, stream>>>(
       (T*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, q_start,
       ctx_len, block_table, bt_stride, work_seq, work_qoff, Hq, Hkv, D, page_size, window, scale);
   return ptl_launch_status();
@@ -167,12 +181,22 @@ extern "C" int ptl_attention_generic(void* out, long out_stride, const void* q, 
                                      int Hq, int Hkv, int D, int page_size, int window, float scale,
                                      int dtype, hipStream_t stream) {
   if (n_work <= 0) return PTL_OK;
-  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || D > 256 || page_size <= 0 ||
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || D > 640 || page_size <= 0 ||
       Hq > 65535)
     return PTL_ERR_ARG;
 #define GO(T, BN) launch_generic<T, BN>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
                                         ctx_len, block_table, bt_stride, work_seq, work_qoff,   \
                                         n_work, Hq, Hkv, D, page_size, window, scale, stream)
+  if (D > 256) {
+    // wide heads (a latent cache of 512 + 64, say): 40 columns a thread, 16 keys a turn
+#define GO_WIDE(T) launch_generic<T, 16, 40>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
+                                             ctx_len, block_table, bt_stride, work_seq, work_qoff,  \
+                                             n_work, Hq, Hkv, D, page_size, window, scale, stream)
+    if (dtype == PTL_DTYPE_F32) return GO_WIDE(float);
+    if (dtype == PTL_DTYPE_BF16) return GO_WIDE(bf16_t);
+#undef GO_WIDE
+    return PTL_ERR_ARG;
+  }
   if (dtype == PTL_DTYPE_F32) return D <= 128 ? GO(float, 32) : GO(float, 16);
   if (dtype == PTL_DTYPE_BF16) return D <= 128 ? GO(bf16_t, 32) : GO(bf16_t, 16);
 #undef GO

@@ -634,8 +634,8 @@ def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[3] != D:
         raise KernelError("attention: caches must be [pages, Hkv, page_size, D]")
     Hkv, page_size = k_cache.shape[1], k_cache.shape[2]
-    if D > 256:
-        raise KernelError(f"attention: head size {D} exceeds the kernel's limit of 256")
+    if D > 640:
+        raise KernelError(f"attention: head size {D} exceeds the kernel's limit of 640")
     if Hq % Hkv:
         raise KernelError(f"attention: {Hq} query heads are not a multiple of {Hkv} kv heads")
     if q.stride(2) != 1 or out.stride(2) != 1 or (Hq > 1 and (q.stride(1) != D or out.stride(1) != D)):

@@ -41,8 +41,8 @@ class PagedAttention(Part):
                  v_name: str = "v_proj.weight", o_name: str = "o_proj.weight"):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
-        if (head_dim % 2 and position is not None) or head_dim > 256:
-            raise ValueError(f"the attention kernels take head sizes up to 256 (even ones with a "
+        if (head_dim % 2 and position is not None) or head_dim > 640:
+            raise ValueError(f"the attention kernels take head sizes up to 640 (even ones with a "
                              f"position encoding), got {head_dim}")
         self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
         self.num_kv_heads, self.head_dim = int(num_kv_heads), int(head_dim)
@@ -174,7 +174,7 @@ class PagedAttention(Part):
         k = cache.k if k is None else k
         v = cache.v if v is None else v
         D, window = self.head_dim, self.window or 0
-        n_dec = ctx.num_decode_seqs if D % 16 == 0 else 0
+        n_dec = ctx.num_decode_seqs if D % 16 == 0 and D <= 256 else 0      # (else: the vector kernel)
         if n_dec:
             mfma = (ops.attention_decode_mfma_fits(q.dtype, self.num_heads, self.num_kv_heads, D,
                                                    cache.page_size)

@@ -45,8 +45,8 @@ class LatentAttention(Part):
         if rot_dim % 2 or rot_dims % 2 or rot_dims > rot_dim:
             raise ValueError(f"rotated size {rot_dim} with {rot_dims} rotating entries: both must be even, "
                              "the second at most the first")
-        if kv_rank + rot_dim > 256:
-            raise ValueError(f"the attention kernels take kv_rank + rot_dim up to 256, got {kv_rank + rot_dim}")
+        if kv_rank + rot_dim > 640:
+            raise ValueError(f"the attention kernels take kv_rank + rot_dim up to 640, got {kv_rank + rot_dim}")
         self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
         self.dim, self.rot_dim, self.vdim, self.kv_rank = int(dim), int(rot_dim), int(vdim), int(kv_rank)
         self.scale, self.eps = float(scale), float(eps)

@@ -89,9 +89,16 @@ def _r5():
     ])
 
 
+def _r6():
+    """A latent as wide as those of the largest public models of this kind (512 + 64): beyond
+    the head sizes of the matrix-core and split-KV kernels, the vector kernel takes it."""
+    m = dict(heads=2, dim=8, rot_dim=64, vdim=8, kv_rank=512, scale=0.1, base=10000.0)
+    return model(100, 64, 2.0, 1e-6, 0, [layer(mixer(**m), dense(48)), layer(mixer(**m, kv_from=0), None)])
+
+
 # name -> (config, weight std, page size)
 RUBASUN = {"R1": (_r1(), 0.12, 16), "R2": (_r2(), 0.10, 4), "R3": (_r3(), 0.10, 8), "R4": (_r4(), 0.15, 16),
-           "R5": (_r5(), 0.15, 8)}
+           "R5": (_r5(), 0.15, 8), "R6": (_r6(), 0.12, 16)}
 
 
 def rubasun(name):
