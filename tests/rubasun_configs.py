@@ -96,9 +96,19 @@ def _r6():
     return model(100, 64, 2.0, 1e-6, 0, [layer(mixer(**m), dense(48)), layer(mixer(**m, kv_from=0), None)])
 
 
+def _r7():
+    """More than 16 heads on a latent size that the matrix-core kernels take (prompt portions on
+    the matrix cores, decoded tokens through the vector split-KV kernel), one expert a token."""
+    m = dict(heads=18, dim=8, rot_dim=32, vdim=8, kv_rank=64, scale=0.12, base=3000.0)
+    return model(150, 96, 5.0, 1e-6, 2, [layer(mixer(**m), moe(7, 1, 24, 1.5, 16, 1.5)),
+                                        layer(mixer(**m, kv_from=0), dense(80)),
+                                        layer(mixer(**m), None)])
+
+
 # name -> (config, weight std, page size)
 RUBASUN = {"R1": (_r1(), 0.12, 16), "R2": (_r2(), 0.10, 4), "R3": (_r3(), 0.10, 8), "R4": (_r4(), 0.15, 16),
-           "R5": (_r5(), 0.15, 8), "R6": (_r6(), 0.12, 16)}
+           "R5": (_r5(), 0.15, 8), "R6": (_r6(), 0.12, 16),
+           "R7": (_r7(), 0.10, 16)}
 
 
 def rubasun(name):

@@ -19,9 +19,9 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LENGTHS = {"R1": [5, 9, 33, 70, 130, 47], "R2": [3, 17, 40, 65, 31], "R3": [12, 50, 90, 20],
-           "R4": [7, 30, 64, 81], "R5": [9, 26, 75, 40], "R6": [20, 70, 33]}
+           "R4": [7, 30, 64, 81], "R5": [9, 26, 75, 40], "R6": [20, 70, 33], "R7": [15, 66, 101, 38]}
 DTYPES = [torch.float32, torch.bfloat16]
-NAMES = ["R1", "R2", "R3", "R4", "R5", "R6"]
+NAMES = ["R1", "R2", "R3", "R4", "R5", "R6", "R7"]
 
 
 def read_folder(folder):
