@@ -137,8 +137,11 @@ class LatentAttention(Part):
         ops.latent_prepare(q, p, 0, self.kv_off, ctx.positions, self.inv_freq, self.c_weight, self.eps,
                            group.slots if (cache.writable and self.own_kv) else None, pool,
                            H, self.dim, dr, R)
-        qn = p[:, :self.q_size].view(T, H, self.dim + dr)[:, :, :self.dim]
-        ops.gemm_heads_nt(q[:, :, :R], qn, self.ukT)
+        if self.dim:
+            qn = p[:, :self.q_size].view(T, H, self.dim + dr)[:, :, :self.dim]
+            ops.gemm_heads_nt(q[:, :, :R], qn, self.ukT)
+        else:                               # (queries without an unrotated part: only kr is matched)
+            q[:, :, :R].zero_()
         lat = torch.empty((T, H, D), dtype=x.dtype, device=x.device)
         self.core.attend(lat, q, cache, ctx, group, k=pool, v=pool)
         out = torch.empty((T, H, self.vdim), dtype=x.dtype, device=x.device)
