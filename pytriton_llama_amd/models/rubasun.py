@@ -67,6 +67,8 @@ def build_rubasun(cfg: RubasunConfig) -> CausalLM:
             schedule.append(LayerCall(i, cache_of[i], True))
         else:
             schedule.append(LayerCall(i, cache_of[m.kv_from], False))
+    for before, after in zip(blocks, blocks[1:]):      # (the run order is the order of the layers)
+        before.next_norm = after.norm1
     final_norm = _norm(cfg)
     head = build_part("head", "linear_head", vocab_size=cfg.vocab_size, hidden_size=W, weight_name="head")
     prefixes = [("", embedding)]

@@ -87,7 +87,12 @@ class SandwichBlock(Part):
     Dynamic-Tanh norms the norm behind a sublayer, the sum and the norm in front of the next
     one are one kernel (ops.stream_add_dyt); other norms run through their own ``forward``
     and a plain sum into the stream. Sublayers read and return the engine's dtype (a
-    feed-forward may return float32)."""
+    feed-forward may return float32).
+
+    ``next_norm`` (set by the model's builder): the Dynamic-Tanh norm in front of the mixer of
+    the block that runs next. The block's last kernel then applies it as well and the second
+    value it returns, where other blocks carry a residual, is the stream normed for that mixer;
+    a block that is handed such a value starts from it instead of norming the stream itself."""
 
     def __init__(self, pre_mixer_norm: Part, mixer: Part, post_mixer_norm: Part,
                  pre_ffn_norm: Part = None, feed_forward: Part = None, post_ffn_norm: Part = None,
@@ -102,6 +107,7 @@ class SandwichBlock(Part):
             libs += tuple(p.kernel_libraries)
         self.kernel_libraries = tuple(dict.fromkeys(libs))
         self.dtype = None
+        self.next_norm = None
 
     def children(self):
         roles = {"norm1": self.norm1, "mixer": self.mixer, "norm1b": self.norm1b, "norm2": self.norm2,
@@ -146,22 +152,28 @@ class SandwichBlock(Part):
         return out, copy
 
     def forward(self, h, residual, ctx, cache):
-        if residual is not None or h.dtype != torch.float32:
-            raise ops.KernelError("a sandwich block runs on a float32 residual stream without a second one")
+        if h.dtype != torch.float32:
+            raise ops.KernelError("a sandwich block runs on a float32 residual stream")
         stream = h
         dtype = self.mixer_dtype()
-        a, _ = self._add(stream, None, None, self.norm1, dtype)
+        if residual is not None:            # the stream, normed for this mixer by the block before
+            a = residual
+        else:
+            a, _ = self._add(stream, None, None, self.norm1, dtype)
         y = self.mixer.forward(a, ctx, cache)
+        nxt = self.next_norm if self._fusable(self.next_norm) else None
         want_copy = self.side is not None and dtype != torch.float32
+        last_pre = None if self.side is not None else nxt
         if self.feed_forward is not None:
             a, _ = self._add(stream, y, self.norm1b, self.norm2, dtype)
             y = self.feed_forward.forward(a)
-            _, copy = self._add(stream, y, self.norm2b, None, dtype, want_copy)
+            ahead, copy = self._add(stream, y, self.norm2b, last_pre, dtype, want_copy)
         else:
-            _, copy = self._add(stream, y, self.norm1b, None, dtype, want_copy)
+            ahead, copy = self._add(stream, y, self.norm1b, last_pre, dtype, want_copy)
         if self.side is not None:
-            self.side.forward(stream, copy if want_copy else stream, ctx.token_ids)
-        return stream, None
+            ahead = self.side.forward(stream, copy if want_copy else stream, ctx.token_ids,
+                                      nxt.params() if nxt is not None else None, dtype)
+        return stream, ahead
 
     def mixer_dtype(self):
         """The engine's dtype, as the parts hold it after loading."""
