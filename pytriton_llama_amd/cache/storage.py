@@ -61,9 +61,13 @@ class CacheStorage:
             shape = (len(g.layers), manager.max_num_seqs + 1) + tuple(g.spec.shape)
             self.state_pools.append(torch.zeros(shape, dtype=g.spec.dtype or dtype, device=device))
 
-    def view(self, cache_layer: Optional[int], writable: bool = True):
+    def view(self, cache_layer, writable: bool = True):
+        """The view of one cache layer, or a tuple of views for a tuple of layers (a mixer made
+        of several, each with a cache of its own kind)."""
         if cache_layer is None:
             return None
+        if isinstance(cache_layer, (tuple, list)):
+            return tuple(self.view(c, writable) for c in cache_layer)
         home = self.manager.layer_home[cache_layer]
         if home is None:
             return None

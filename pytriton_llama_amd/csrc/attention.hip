@@ -25,20 +25,25 @@
 
 #define BM 16
 
-// NJ: head-size columns a thread accumulates, 16 apart (16: head sizes up to 256; 40: up to 640)
-template <typename T, int BN, int NJ = 16>
+// NJ: value columns a thread accumulates, 16 apart (16: value sizes up to 256; 40: up to 640).
+// Keys of size Dk and values of size Dv need not be alike, and a query head may come in
+// ``maps`` forms (several score maps over one set of values): query head j is map j % maps of
+// head j / maps, reads key head (kv head) * maps + j % maps and value head (kv head), with
+// kv head = (j / maps) / (heads a kv head). TO: the type of the result (T, or float for a
+// result that is combined further before it is rounded).
+template <typename T, typename TO, int BN, int NJ = 16>
 __global__ void __launch_bounds__(256)
-attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q, long q_stride,
+attn_generic_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__ q, long q_stride,
                     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
                     const int32_t* __restrict__ block_table, int bt_stride,
                     const int32_t* __restrict__ work_seq, const int32_t* __restrict__ work_qoff,
-                    int Hq, int Hkv, int D, int page_size, int window, float scale) {
+                    int Hq, int Hkv, int maps, int Dk, int Dv, int page_size, int window, float scale) {
   extern __shared__ float lds[];
-  float* Qs = lds;                   // [BM][D]
-  float* Ks = Qs + BM * D;           // [BN][D+1]
-  float* Vs = Ks + BN * (D + 1);     // [BN][D]
-  float* Ss = Vs + BN * D;           // [BM][BN]
+  float* Qs = lds;                   // [BM][Dk]
+  float* Ks = Qs + BM * Dk;          // [BN][Dk+1]
+  float* Vs = Ks + BN * (Dk + 1);    // [BN][Dv]
+  float* Ss = Vs + BN * Dv;          // [BM][BN]
 
   const int tid = threadIdx.x;
   const int head = blockIdx.y;
@@ -50,12 +55,14 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
   const int cached = ctx - qlen;
   const int rows = min(BM, qlen - qoff);
   if (rows <= 0) return;
-  const int kvh = head / (Hq / Hkv);
+  const int vh = (head / maps) / ((Hq / maps) / Hkv);      // value head
+  const int kh = vh * maps + head % maps;                   // key head (of Hkv * maps)
+  const int Hk = Hkv * maps;
   const int32_t* bt = block_table + (size_t)seq * bt_stride;
 
-  for (int i = tid; i < BM * D; i += 256) {
-    const int m = i / D, d = i - m * D;
-    Qs[i] = m < rows ? to_float<T>(q[(size_t)(qs + qoff + m) * q_stride + head * D + d]) : 0.f;
+  for (int i = tid; i < BM * Dk; i += 256) {
+    const int m = i / Dk, d = i - m * Dk;
+    Qs[i] = m < rows ? to_float<T>(q[(size_t)(qs + qoff + m) * q_stride + head * Dk + d]) : 0.f;
   }
 
   const int tm = tid >> 4, tc = tid & 15;
@@ -65,7 +72,7 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
   const int k_end = min(ctx, first_q + rows);
   const int k_lo = window > 0 ? max(0, first_q - window + 1) : 0;
   const int k_begin = (k_lo / BN) * BN;
-  const int nd = (D + 15) >> 4;
+  const int nd = (Dv + 15) >> 4;
 
   float m_run = -INFINITY, l_run = 0.f;
   float acc[NJ];
@@ -74,20 +81,27 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
 
   for (int k0 = k_begin; k0 < k_end; k0 += BN) {
     __syncthreads();
-    for (int i = tid; i < BN * D; i += 256) {
-      const int n = i / D, d = i - n * D;
+    for (int i = tid; i < BN * Dk; i += 256) {
+      const int n = i / Dk, d = i - n * Dk;
       const int kp = k0 + n;
-      float kv = 0.f, vv = 0.f;
+      float kv = 0.f;
       if (kp >= k_lo && kp < k_end) {
         const int page = bt[kp / page_size];
-        if (page >= 0) {
-          const size_t idx = (((size_t)page * Hkv + kvh) * page_size + (kp % page_size)) * D + d;
-          kv = to_float<T>(k_cache[idx]);
-          vv = to_float<T>(v_cache[idx]);
-        }
+        if (page >= 0)
+          kv = to_float<T>(k_cache[(((size_t)page * Hk + kh) * page_size + (kp % page_size)) * Dk + d]);
       }
-      Ks[n * (D + 1) + d] = kv;
-      Vs[n * D + d] = vv;
+      Ks[n * (Dk + 1) + d] = kv;
+    }
+    for (int i = tid; i < BN * Dv; i += 256) {
+      const int n = i / Dv, d = i - n * Dv;
+      const int kp = k0 + n;
+      float vv = 0.f;
+      if (kp >= k_lo && kp < k_end) {
+        const int page = bt[kp / page_size];
+        if (page >= 0)
+          vv = to_float<T>(v_cache[(((size_t)page * Hkv + vh) * page_size + (kp % page_size)) * Dv + d]);
+      }
+      Vs[i] = vv;
     }
     __syncthreads();
 
@@ -97,10 +111,10 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
     for (int j = 0; j < BN / 16; ++j) {
       const int n = tc + 16 * j;
       const int kp = k0 + n;
-      const float* qr = Qs + tm * D;
-      const float* kr = Ks + n * (D + 1);
+      const float* qr = Qs + tm * Dk;
+      const float* kr = Ks + n * (Dk + 1);
       float dot = 0.f;
-      for (int d = 0; d < D; ++d) dot = fmaf(qr[d], kr[d], dot);
+      for (int d = 0; d < Dk; ++d) dot = fmaf(qr[d], kr[d], dot);
       const bool vis = row_valid && kp <= qpos && kp < ctx && (window <= 0 || kp > qpos - window);
       s[j] = vis ? dot * scale : -INFINITY;
       tmax = fmaxf(tmax, s[j]);
@@ -128,35 +142,35 @@ attn_generic_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ 
     const int n_lim = min(BN, k_end - k0);
     for (int n = 0; n < n_lim; ++n) {
       const float p = Ss[tm * BN + n];
-      const float* vr = Vs + n * D + tc;
+      const float* vr = Vs + n * Dv + tc;
 #pragma unroll
       for (int j = 0; j < NJ; ++j)
-        if (j < nd && tc + 16 * j < D) acc[j] = fmaf(p, vr[16 * j], acc[j]);
+        if (j < nd && tc + 16 * j < Dv) acc[j] = fmaf(p, vr[16 * j], acc[j]);
     }
   }
 
   if (row_valid) {
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-    T* o = out + (size_t)(qs + qoff + tm) * out_stride + head * D + tc;
+    TO* o = out + (size_t)(qs + qoff + tm) * out_stride + head * Dv + tc;
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
-      if (j < nd && tc + 16 * j < D) o[16 * j] = from_float<T>(acc[j] * inv);
+      if (j < nd && tc + 16 * j < Dv) o[16 * j] = from_float<TO>(acc[j] * inv);
   }
 }
 
-template <typename T, int BN, int NJ = 16>
+template <typename T, typename TO, int BN, int NJ = 16>
 static int launch_generic(void* out, long out_stride, const void* q, long q_stride,
                           const void* k_cache, const void* v_cache, const int32_t* q_start,
                           const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
                           const int32_t* work_seq, const int32_t* work_qoff, int n_work,
-                          int Hq, int Hkv, int D, int page_size, int window, float scale,
-                          hipStream_t stream) {
-  const size_t lds = (size_t)(BM * D + BN * (D + 1) + BN * D + BM * BN) * sizeof(float);
+                          int Hq, int Hkv, int maps, int Dk, int Dv, int page_size, int window,
+                          float scale, hipStream_t stream) {
+  const size_t lds = (size_t)(BM * Dk + BN * (Dk + 1) + BN * Dv + BM * BN) * sizeof(float);
   if (lds > 64 * 1024) {
     // more dynamic LDS than a kernel may ask for without saying so beforehand (wide heads only)
     static size_t allowed = 0;
     if (lds > allowed) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_generic_kernel<T, BN, NJ>),
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_generic_kernel<T, TO, BN, NJ>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return PTL_ERR_ARG;
@@ -165,14 +179,49 @@ static int launch_generic(void* out, long out_stride, const void* q, long q_stri
     }
   }
   dim3 grid(n_work, Hq);
-  attn_generic_kernel<T, BN, NJ><<<grid, 256, lds, stream>>>(
-      (T*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, q_start,
-      ctx_len, block_table, bt_stride, work_seq, work_qoff, Hq, Hkv, D, page_size, window, scale);
+  attn_generic_kernel<T, TO, BN, NJ><<<grid, 256, lds, stream>>>(
+      (TO*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, q_start,
+      ctx_len, block_table, bt_stride, work_seq, work_qoff, Hq, Hkv, maps, Dk, Dv, page_size, window,
+      scale);
   return ptl_launch_status();
 }
 
-// work_seq / work_qoff list the 16-row query blocks: block i covers rows
+// The general form. q [T, Hq, Dk] with Hq = heads * maps; k_cache [pages, Hkv * maps, page_size,
+// Dk]; v_cache [pages, Hkv, page_size, Dv]; out [T, Hq, Dv] of the caches' type, or float32 when
+// out_f32 is set. work_seq / work_qoff list the 16-row query blocks: block i covers rows
 // work_qoff[i] .. work_qoff[i]+15 of sequence work_seq[i].
+extern "C" int ptl_attention_generic_kv(void* out, long out_stride, int out_f32, const void* q,
+                                        long q_stride, const void* k_cache, const void* v_cache,
+                                        const int32_t* q_start, const int32_t* ctx_len,
+                                        const int32_t* block_table, int bt_stride,
+                                        const int32_t* work_seq, const int32_t* work_qoff, int n_work,
+                                        int Hq, int Hkv, int maps, int Dk, int Dv, int page_size,
+                                        int window, float scale, int dtype, hipStream_t stream) {
+  if (n_work <= 0) return PTL_OK;
+  if (Hq <= 0 || Hkv <= 0 || maps <= 0 || Hq % maps || (Hq / maps) % Hkv || Dk <= 0 || Dv <= 0 ||
+      Dk > 640 || Dv > 640 || page_size <= 0 || Hq > 65535)
+    return PTL_ERR_ARG;
+#define GO(T, TO, BN, NJ)                                                                         \
+  launch_generic<T, TO, BN, NJ>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len, \
+                                block_table, bt_stride, work_seq, work_qoff, n_work, Hq, Hkv,    \
+                                maps, Dk, Dv, page_size, window, scale, stream)
+#define GO_SIZES(T, TO)                                                                           \
+  {                                                                                               \
+    /* wide heads (a latent cache of 512 + 64, say): 40 columns a thread, 16 keys a turn */       \
+    if (Dk > 256 || Dv > 256) return GO(T, TO, 16, 40);                                           \
+    return (Dk <= 128 && Dv <= 128) ? GO(T, TO, 32, 16) : GO(T, TO, 16, 16);                      \
+  }
+  if (dtype == PTL_DTYPE_F32) GO_SIZES(float, float)
+  if (dtype == PTL_DTYPE_BF16) {
+    if (out_f32) GO_SIZES(bf16_t, float)
+    GO_SIZES(bf16_t, bf16_t)
+  }
+#undef GO_SIZES
+#undef GO
+  return PTL_ERR_ARG;
+}
+
+// Keys and values of one size, one score map a head.
 extern "C" int ptl_attention_generic(void* out, long out_stride, const void* q, long q_stride,
                                      const void* k_cache, const void* v_cache,
                                      const int32_t* q_start, const int32_t* ctx_len,
@@ -180,27 +229,9 @@ extern "C" int ptl_attention_generic(void* out, long out_stride, const void* q, 
                                      const int32_t* work_seq, const int32_t* work_qoff, int n_work,
                                      int Hq, int Hkv, int D, int page_size, int window, float scale,
                                      int dtype, hipStream_t stream) {
-  if (n_work <= 0) return PTL_OK;
-  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || D > 640 || page_size <= 0 ||
-      Hq > 65535)
-    return PTL_ERR_ARG;
-#define GO(T, BN) launch_generic<T, BN>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
-                                        ctx_len, block_table, bt_stride, work_seq, work_qoff,   \
-                                        n_work, Hq, Hkv, D, page_size, window, scale, stream)
-  if (D > 256) {
-    // wide heads (a latent cache of 512 + 64, say): 40 columns a thread, 16 keys a turn
-#define GO_WIDE(T) launch_generic<T, 16, 40>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
-                                             ctx_len, block_table, bt_stride, work_seq, work_qoff,  \
-                                             n_work, Hq, Hkv, D, page_size, window, scale, stream)
-    if (dtype == PTL_DTYPE_F32) return GO_WIDE(float);
-    if (dtype == PTL_DTYPE_BF16) return GO_WIDE(bf16_t);
-#undef GO_WIDE
-    return PTL_ERR_ARG;
-  }
-  if (dtype == PTL_DTYPE_F32) return D <= 128 ? GO(float, 32) : GO(float, 16);
-  if (dtype == PTL_DTYPE_BF16) return D <= 128 ? GO(bf16_t, 32) : GO(bf16_t, 16);
-#undef GO
-  return PTL_ERR_ARG;
+  return ptl_attention_generic_kv(out, out_stride, 0, q, q_stride, k_cache, v_cache, q_start, ctx_len,
+                                  block_table, bt_stride, work_seq, work_qoff, n_work, Hq, Hkv, 1, D,
+                                  D, page_size, window, scale, dtype, stream);
 }
 
 // ===========================================================================

@@ -1,0 +1,327 @@
+// Mixers that carry a matrix of fixed size from token to token instead of a cache that grows.
+// Per head a matrix S [D, Dv] (keys x values), float32, kept in the request's state slot:
+//
+//   gated delta rule:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//   matrix memory:     m' = max(f + m, i);  S <- e^(f + m - m') S + e^(i - m') k v^T;
+//                      n <- e^(f + m - m') n + e^(i - m') k;
+//                      o = S^T q / (max(|n . q|, e^(-m')) + 1e-6)           (m starts at 0)
+//
+// Every column of S (one value entry) goes its own way given k, q and the gates, so the columns
+// are spread over the chip: a workgroup takes 16 columns of one head of one sequence, a column is
+// held by 16 lanes (one row of a wave for the data-parallel lane moves), each lane with R rows of it
+// in registers (D <= 16 R; rows beyond D stay zero). A step is R multiply-adds for each product
+// and a sum over the 16 lanes; the tokens of a sequence are walked in order, 16 at a time through
+// LDS, so the result does not depend on how the sequence was cut into steps. n and m of the
+// matrix memory are kept once per column block (every block carries the same values), so that no
+// workgroup reads what another one writes.
+//
+// State of a slot: [H][blocks of 16 columns][16 D + D + 4] floats: S^T of the block (column
+// after column, D rows each), then n [D], then m (matrix memory only; the delta rule leaves both
+// untouched). The delta rule's slot also holds, behind that, the last taps - 1 inputs of its short
+// convolutions [taps - 1][C].
+//
+// ptl_conv_prepare: for every token and head the short causal convolution over time of q, k and v
+//   (inputs before the step's first token come from the slot), SiLU, and for q and k the unit norm
+//   x / sqrt(sum(x^2) + 1e-6) (q also times D^-1/2), all float32.
+// ptl_conv_tail_update: afterwards, the slot's last taps - 1 inputs.
+// ptl_delta_scan / ptl_memory_scan: the recurrences; gates from the float32 projection.
+#include "common.h"
+#include <math.h>
+
+#define CHUNK 16
+
+__device__ __forceinline__ float row16_sum(float v) {
+  // the sum over the 16 lanes of a row, in every lane: rotations by 8, 4, 2 and 1 inside the row
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
+  return v;
+}
+
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+__device__ __forceinline__ float logsigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+#define MODE_DELTA 0
+#define MODE_MEMORY 1
+
+struct ScanArgs {
+  float* out;            // [T, H, Dv]
+  const float* q; long ldq;      // q[t * ldq + g * D + d]
+  const float* k; long ldk;
+  const float* v; long ldv;      // v[t * ldv + h * Dv + c]
+  const float* ga; const float* gb; long ldg;   // raw gates [t * ldg + h]: delta (a, b); memory (i, f)
+  const float* c0; const float* c1;              // [H]: delta (A_log, dt_bias); memory (i bias, f bias)
+  float cap, qscale;
+  float* state; long slot_stride;
+  const int32_t* q_start; const int32_t* state_slots;
+  int H, heads_per_qk, D, Dv;
+};
+
+template <int R, int MODE>
+__global__ void __launch_bounds__(256) scan_kernel(ScanArgs A) {
+  constexpr int DP = 16 * R;
+  __shared__ float ks[CHUNK][DP], qs[CHUNK][DP], vs[CHUNK][16], os[CHUNK][16], g0s[CHUNK], g1s[CHUNK];
+  const int tid = threadIdx.x;
+  const int b = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
+  const int row0 = A.q_start[seq];
+  const int qlen = A.q_start[seq + 1] - row0;
+  if (qlen <= 0) return;
+  const int D = A.D, Dv = A.Dv;
+  const int slot = A.state_slots[seq];
+  const int nb = (Dv + 15) >> 4;
+  const int block_floats = 16 * D + D + 4;
+  float* st = A.state + (size_t)slot * A.slot_stride + ((size_t)h * nb + b) * block_floats;
+  const int cg = tid >> 4, l = tid & 15;           // column of the block, lane of the column
+  const int col = b * 16 + cg;
+  const int g = h / A.heads_per_qk;
+  float S[R], n[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int d = l * R + r;
+    S[r] = (d < D && col < Dv) ? st[(size_t)cg * D + d] : 0.f;
+    n[r] = (MODE == MODE_MEMORY && d < D) ? st[16 * D + d] : 0.f;
+  }
+  float m = MODE == MODE_MEMORY ? st[16 * D + D] : 0.f;
+
+  for (int t0 = 0; t0 < qlen; t0 += CHUNK) {
+    const int steps = min(CHUNK, qlen - t0);
+    __syncthreads();
+    for (int i = tid; i < CHUNK * DP; i += 256) {
+      const int t = i / DP, d = i - t * DP;
+      float kv = 0.f, qv = 0.f;
+      if (t < steps && d < D) {
+        const size_t row = (size_t)(row0 + t0 + t);
+        kv = A.k[row * A.ldk + (size_t)g * D + d];
+        qv = A.q[row * A.ldq + (size_t)g * D + d] * A.qscale;
+      }
+      ks[t][d] = kv;
+      qs[t][d] = qv;
+    }
+    {
+      const int t = tid >> 4, c = tid & 15;          // (256 threads: CHUNK x 16)
+      const int cc = b * 16 + c;
+      vs[t][c] = (t < steps && cc < Dv) ? A.v[(size_t)(row0 + t0 + t) * A.ldv + (size_t)h * Dv + cc] : 0.f;
+    }
+    if (tid < steps) {
+      const size_t row = (size_t)(row0 + t0 + tid);
+      const float a = A.ga[row * A.ldg + h], bb = A.gb[row * A.ldg + h];
+      if (MODE == MODE_DELTA) {
+        g0s[tid] = expf(-expf(A.c0[h]) * softplus_f(a + A.c1[h]));      // decay
+        g1s[tid] = 1.0f / (1.0f + expf(-bb));                            // beta
+      } else {
+        g0s[tid] = A.cap * tanhf((a + A.c0[h]) / A.cap);                 // log input gate
+        g1s[tid] = logsigmoid_f(A.cap * tanhf((bb + A.c1[h]) / A.cap));  // log forget gate
+      }
+    }
+    __syncthreads();
+    for (int t = 0; t < steps; ++t) {
+      float kr[R], qr[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        kr[r] = ks[t][l * R + r];
+        qr[r] = qs[t][l * R + r];
+      }
+      const float v = vs[t][cg];
+      float o;
+      if (MODE == MODE_DELTA) {
+        const float decay = g0s[t], beta = g1s[t];
+        float sk = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] *= decay;
+          sk = fmaf(S[r], kr[r], sk);
+        }
+        sk = row16_sum(sk);
+        const float u = beta * (v - sk);
+        float sq = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] = fmaf(kr[r], u, S[r]);
+          sq = fmaf(S[r], qr[r], sq);
+        }
+        o = row16_sum(sq);
+      } else {
+        const float gi = g0s[t], gf = g1s[t];
+        const float m_new = fmaxf(gf + m, gi);
+        const float keep = expf(gf + m - m_new), take = expf(gi - m_new);
+        m = m_new;
+        const float tv = take * v;
+        float sq = 0.f, nq = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] = fmaf(kr[r], tv, keep * S[r]);
+          n[r] = fmaf(kr[r], take, keep * n[r]);
+          sq = fmaf(S[r], qr[r], sq);
+          nq = fmaf(n[r], qr[r], nq);
+        }
+        sq = row16_sum(sq);
+        nq = row16_sum(nq);
+        o = sq / (fmaxf(fabsf(nq), expf(-m_new)) + 1e-6f);
+      }
+      if (l == 0) os[t][cg] = o;
+    }
+    __syncthreads();
+    {
+      const int t = tid >> 4, c = tid & 15;
+      const int cc = b * 16 + c;
+      if (t < steps && cc < Dv) A.out[((size_t)(row0 + t0 + t) * A.H + h) * Dv + cc] = os[t][c];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int d = l * R + r;
+    if (d < D && col < Dv) st[(size_t)cg * D + d] = S[r];
+    if (MODE == MODE_MEMORY && cg == 0 && d < D) st[16 * D + d] = n[r];
+  }
+  if (MODE == MODE_MEMORY && tid == 0) st[16 * D + D] = m;
+}
+
+template <int MODE>
+static int launch_scan(const ScanArgs& A, int n_seqs, hipStream_t st) {
+  const int nb = (A.Dv + 15) / 16;
+  if (A.D <= 0 || A.D > 256 || A.Dv <= 0 || A.H <= 0 || A.H > 65535 || n_seqs > 65535 ||
+      A.heads_per_qk <= 0 || A.H % A.heads_per_qk)
+    return PTL_ERR_ARG;
+  dim3 grid(nb, A.H, n_seqs);
+  const int R = (A.D + 15) / 16;
+#define GO(RR)                                            \
+  if (R <= RR) {                                          \
+    scan_kernel<RR, MODE><<<grid, 256, 0, st>>>(A);       \
+    return ptl_launch_status();                           \
+  }
+  GO(1) GO(2) GO(3) GO(4) GO(6) GO(8) GO(12) GO(16)
+#undef GO
+  return PTL_ERR_ARG;
+}
+
+// q, k float32 [T, G, D] (unit vectors), v float32 [T, H, Dv]; raw gates a and b float32 with row
+// stride ldg, one a head; A_log, dt_bias float32 [H]. state: the slots, slot_stride floats each.
+extern "C" int ptl_delta_scan(float* out, const float* q, const float* k, const float* v, const float* ga,
+                              const float* gb, long ldg, const float* A_log, const float* dt_bias,
+                              float* state, long slot_stride, const int32_t* q_start,
+                              const int32_t* state_slots, int n_seqs, int H, int G, int D, int Dv,
+                              hipStream_t st) {
+  if (n_seqs <= 0) return PTL_OK;
+  if (G <= 0 || H % G) return PTL_ERR_ARG;
+  ScanArgs A{out, q, (long)G * D, k, (long)G * D, v, (long)H * Dv, ga, gb, ldg, A_log, dt_bias, 0.f, 1.f,
+             state, slot_stride, q_start, state_slots, H, H / G, D, Dv};
+  return launch_scan<MODE_DELTA>(A, n_seqs, st);
+}
+
+// q, k, v: columns of the float32 projection p [T, ldp] (H heads of D, D and Dv); raw gates i and f
+// at columns i_off and f_off, their biases float32 [H]; q is multiplied by qscale.
+extern "C" int ptl_memory_scan(float* out, const float* p, long ldp, int q_off, int k_off, int v_off,
+                               int i_off, int f_off, const float* i_bias, const float* f_bias, float cap,
+                               float qscale, float* state, long slot_stride, const int32_t* q_start,
+                               const int32_t* state_slots, int n_seqs, int H, int D, int Dv,
+                               hipStream_t st) {
+  if (n_seqs <= 0) return PTL_OK;
+  if (cap <= 0.f) return PTL_ERR_ARG;
+  ScanArgs A{out, p + q_off, ldp, p + k_off, ldp, p + v_off, ldp, p + i_off, p + f_off, ldp, i_bias, f_bias,
+             cap, qscale, state, slot_stride, q_start, state_slots, H, 1, D, Dv};
+  return launch_scan<MODE_MEMORY>(A, n_seqs, st);
+}
+
+// ---- the short convolutions in front of the delta rule -------------------------------------------
+__device__ __forceinline__ int seq_of_row(const int32_t* __restrict__ q_start, int n_seqs, int t) {
+  // the last sequence whose first row is not beyond t (sequences without rows share their start
+  // with the one behind them); n_seqs for a row behind all sequences
+  int lo = 0, hi = n_seqs;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (q_start[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+__global__ void __launch_bounds__(256)
+conv_prepare_kernel(float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vv,
+                    const float* __restrict__ p, long ldp, int x_off, const float* __restrict__ cw, int taps,
+                    const float* __restrict__ state, long slot_stride, long tail_off,
+                    const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots, int n_seqs,
+                    int G, int H, int D, int Dv, float qscale) {
+  extern __shared__ float buf[];
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, blk = blockIdx.y, tid = threadIdx.x;
+  const int C = 2 * G * D + H * Dv;
+  const int seq = seq_of_row(q_start, n_seqs, t);
+  int c0, n;
+  float* dst;
+  if (blk < G) { c0 = blk * D; n = D; dst = qn + ((size_t)t * G + blk) * D; }
+  else if (blk < 2 * G) { c0 = G * D + (blk - G) * D; n = D; dst = kn + ((size_t)t * G + (blk - G)) * D; }
+  else { c0 = 2 * G * D + (blk - 2 * G) * Dv; n = Dv; dst = vv + ((size_t)t * H + (blk - 2 * G)) * Dv; }
+  if (seq >= n_seqs) {                      // a row that belongs to no sequence (padding)
+    for (int d = tid; d < n; d += 256) dst[d] = 0.f;
+    return;
+  }
+  const int row0 = q_start[seq];
+  const int r = t - row0;
+  const float* tail = state + (size_t)state_slots[seq] * slot_stride + tail_off;
+  float ss = 0.f;
+  for (int d = tid; d < n; d += 256) {
+    const int c = c0 + d;
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int i = r - (taps - 1) + j;
+      const float x = i >= 0 ? p[(size_t)(row0 + i) * ldp + x_off + c] : tail[(size_t)(taps - 1 + i) * C + c];
+      acc = fmaf(cw[(size_t)c * taps + j], x, acc);
+    }
+    const float y = acc / (1.0f + expf(-acc));
+    buf[d] = y;
+    ss = fmaf(y, y, ss);
+  }
+  if (blk >= 2 * G) {
+    for (int d = tid; d < n; d += 256) dst[d] = buf[d];      // (each thread reads what it wrote)
+    return;
+  }
+  ss = block_sum(ss, scratch);
+  const float sc = (blk < G ? qscale : 1.f) / sqrtf(ss + 1e-6f);
+  for (int d = tid; d < n; d += 256) dst[d] = buf[d] * sc;
+}
+
+// p float32 [T, ldp] with the inputs of the convolutions at columns x_off .. x_off + C, C = 2 G D +
+// H Dv in the order q | k | v; cw float32 [C, taps]; the slot's tail [taps - 1, C] at tail_off.
+extern "C" int ptl_conv_prepare(float* qn, float* kn, float* vv, const float* p, long ldp, int x_off,
+                                const float* cw, int taps, const float* state, long slot_stride,
+                                long tail_off, const int32_t* q_start, const int32_t* state_slots,
+                                int n_seqs, int T_, int G, int H, int D, int Dv, float qscale,
+                                hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (G <= 0 || H <= 0 || D <= 0 || Dv <= 0 || taps <= 0 || n_seqs <= 0 || 2 * G + H > 65535)
+    return PTL_ERR_ARG;
+  const size_t lds = (size_t)(D > Dv ? D : Dv) * sizeof(float);
+  if (lds > 48 * 1024) return PTL_ERR_ARG;
+  dim3 grid(T_, 2 * G + H);
+  conv_prepare_kernel<<<grid, 256, lds, st>>>(qn, kn, vv, p, ldp, x_off, cw, taps, state, slot_stride,
+                                               tail_off, q_start, state_slots, n_seqs, G, H, D, Dv, qscale);
+  return ptl_launch_status();
+}
+
+__global__ void __launch_bounds__(256)
+conv_tail_kernel(float* __restrict__ state, long slot_stride, long tail_off, const float* __restrict__ p,
+                 long ldp, int x_off, const int32_t* __restrict__ q_start,
+                 const int32_t* __restrict__ state_slots, int C, int taps) {
+  const int seq = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int row0 = q_start[seq];
+  const int qlen = q_start[seq + 1] - row0;
+  if (qlen <= 0 || c >= C) return;
+  float* tail = state + (size_t)state_slots[seq] * slot_stride + tail_off;
+  // in order of rising i: an entry read from the old tail lies above the one being written
+  for (int i = 0; i < taps - 1; ++i) {
+    const int r = qlen - (taps - 1) + i;
+    tail[(size_t)i * C + c] = r >= 0 ? p[(size_t)(row0 + r) * ldp + x_off + c] : tail[(size_t)(i + qlen) * C + c];
+  }
+}
+
+extern "C" int ptl_conv_tail_update(float* state, long slot_stride, long tail_off, const float* p, long ldp,
+                                    int x_off, const int32_t* q_start, const int32_t* state_slots,
+                                    int n_seqs, int C, int taps, hipStream_t st) {
+  if (n_seqs <= 0 || taps <= 1) return PTL_OK;
+  if (C <= 0 || n_seqs > 65535) return PTL_ERR_ARG;
+  dim3 grid((C + 255) / 256, n_seqs);
+  conv_tail_kernel<<<grid, 256, 0, st>>>(state, slot_stride, tail_off, p, ldp, x_off, q_start, state_slots,
+                                          C, taps);
+  return ptl_launch_status();
+}

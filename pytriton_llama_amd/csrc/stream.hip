@@ -9,6 +9,8 @@
 //   is optional: no y (only the norm in front), no post norm (a plain sum), no out, and a copy
 //   of the new stream in the engine's dtype for a product that reads the stream itself.
 // ptl_stream_add_rmsnorm: stream += rmsnorm(y) * w, the same with a norm that needs the row.
+// ptl_stream_add_rmsnorm_sum: the same for a result that is a weighted sum of two and a bias.
+// ptl_stream_rmsnorm: the RMS norm of rows of the stream, in the engine's type.
 // ptl_dyt: the norm alone, for rows that are no stream (the rows picked for the head).
 // ptl_embedding_scaled: stream[t] = table[ids[t]] * scale, in float32.
 // ptl_gelu_gather_mul: out[t, j] = gelu_tanh(z[t, j]) * table[ids[t], col0 + j]: a gate on a
@@ -146,6 +148,81 @@ extern "C" int ptl_stream_add_rmsnorm(float* stream, const void* y, int y_dtype,
   if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_F32) GO(bf16_t, float);
 #undef GO
   return PTL_ERR_ARG;
+}
+
+// The same for a sublayer whose result is a weighted sum that has not been added up yet:
+// y = a y1 + b y2 + c bias (y2 and bias optional), stream += rmsnorm(y) * w. The sum is float32.
+template <typename TY, typename TO>
+__global__ void __launch_bounds__(256)
+stream_add_rmsnorm_sum_kernel(float* __restrict__ stream, const TY* __restrict__ y1, float a,
+                              const TY* __restrict__ y2, float b, const float* __restrict__ bias, float c,
+                              const float* __restrict__ w, float eps, TO* __restrict__ copy, int H) {
+  __shared__ float scratch[16];
+  const size_t row = (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < H; j += 256) {
+    float v = a * to_float<TY>(y1[row + j]);
+    if (y2) v = fmaf(b, to_float<TY>(y2[row + j]), v);
+    if (bias) v = fmaf(c, bias[j], v);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int j = threadIdx.x; j < H; j += 256) {
+    float v = a * to_float<TY>(y1[row + j]);
+    if (y2) v = fmaf(b, to_float<TY>(y2[row + j]), v);
+    if (bias) v = fmaf(c, bias[j], v);
+    const float s = stream[row + j] + v * r * w[j];
+    stream[row + j] = s;
+    if (copy) copy[row + j] = from_float<TO>(s);
+  }
+}
+
+extern "C" int ptl_stream_add_rmsnorm_sum(float* stream, const void* y1, float a, const void* y2, float b,
+                                          int y_dtype, const float* bias, float c, const float* w, float eps,
+                                          void* copy, int out_dtype, int T_, int H, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || !stream || !y1 || !w) return PTL_ERR_ARG;
+#define GO(TY, TO)                                                                                    \
+  {                                                                                                   \
+    stream_add_rmsnorm_sum_kernel<TY, TO><<<T_, 256, 0, st>>>(stream, (const TY*)y1, a, (const TY*)y2, b, \
+                                                              bias, c, w, eps, (TO*)copy, H);         \
+    return ptl_launch_status();                                                                       \
+  }
+  if (y_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_F32) GO(float, float);
+  if (y_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_BF16) GO(float, bf16_t);
+  if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_BF16) GO(bf16_t, bf16_t);
+  if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_F32) GO(bf16_t, float);
+#undef GO
+  return PTL_ERR_ARG;
+}
+
+// out = x * rsqrt(mean(x^2) + eps) * w for rows of a float32 stream, in the engine's type (the rows
+// picked for the head).
+template <typename TO>
+__global__ void __launch_bounds__(256)
+stream_rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+                      float eps, int H) {
+  __shared__ float scratch[16];
+  const size_t row = (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < H; j += 256) ss = fmaf(x[row + j], x[row + j], ss);
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int j = threadIdx.x; j < H; j += 256) out[row + j] = from_float<TO>(x[row + j] * r * w[j]);
+}
+
+extern "C" int ptl_stream_rmsnorm(void* out, int out_dtype, const float* x, const float* w, float eps,
+                                  int T_, int H, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || !x || !w) return PTL_ERR_ARG;
+  if (out_dtype == PTL_DTYPE_F32)
+    stream_rmsnorm_kernel<float><<<T_, 256, 0, st>>>((float*)out, x, w, eps, H);
+  else if (out_dtype == PTL_DTYPE_BF16)
+    stream_rmsnorm_kernel<bf16_t><<<T_, 256, 0, st>>>((bf16_t*)out, x, w, eps, H);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
 }
 
 template <typename T>

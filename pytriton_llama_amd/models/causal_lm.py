@@ -21,11 +21,13 @@ def _numel(shape) -> int:
 @dataclass(frozen=True)
 class LayerCall:
     """One entry of the run order: run ``block`` with cache layer
-    ``cache_layer`` (None: the block keeps nothing). ``writes`` False lets a
-    block read a cache layer that another call fills. A block, and a cache
-    layer, may be named by several calls."""
+    ``cache_layer`` (None: the block keeps nothing; a tuple: the block's mixer
+    is made of several mixers and each gets the layer at its place, None for
+    one that keeps nothing). ``writes`` False lets a block read a cache layer
+    that another call fills. A block, and a cache layer, may be named by
+    several calls."""
     block: int
-    cache_layer: Optional[int]
+    cache_layer: object
     writes: bool = True
 
 
@@ -52,9 +54,10 @@ class CausalLM:
         for call in self.schedule:
             if not 0 <= call.block < len(self.blocks):
                 raise ValueError(f"run order names block {call.block}, there are {len(self.blocks)}")
-            if call.cache_layer is not None and not 0 <= call.cache_layer < len(self.cache_layers):
-                raise ValueError(f"run order names cache layer {call.cache_layer}, "
-                                 f"there are {len(self.cache_layers)}")
+            named = call.cache_layer if isinstance(call.cache_layer, (tuple, list)) else (call.cache_layer,)
+            for c in named:
+                if c is not None and not 0 <= c < len(self.cache_layers):
+                    raise ValueError(f"run order names cache layer {c}, there are {len(self.cache_layers)}")
         self.dtype: Optional[torch.dtype] = None
         self.device = None
         self.has_decode_copies = False

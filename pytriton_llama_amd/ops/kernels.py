@@ -1102,6 +1102,301 @@ def gemm_heads_nt(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor,
 
 
 # ---------------------------------------------------------------------------
+# Attention with keys and values of different sizes and several score maps a head
+def attention_generic_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                         q_start: torch.Tensor, ctx_len: torch.Tensor, block_table: torch.Tensor,
+                         work_seq: torch.Tensor, work_qoff: torch.Tensor, scale: float, maps: int = 1,
+                         window: int = 0) -> None:
+    """The vector-FMA attention kernel in its general form (csrc/attention.hip): q [T, Hq, Dk]
+    with Hq = heads * maps (head after head, map after map), k_cache [pages, Hkv * maps, page_size,
+    Dk], v_cache [pages, Hkv, page_size, Dv], out [T, Hq, Dv] in the caches' dtype or float32.
+    Query head j reads key head (its kv head) * maps + j % maps and the values of its kv head."""
+    _need_gpu(out, q, k_cache, v_cache, q_start, ctx_len, block_table, work_seq, work_qoff)
+    if q.dim() != 3 or k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelError("attention: q [T, Hq, Dk], caches [pages, heads, page_size, size]")
+    T, Hq, Dk = q.shape
+    pages, Hk, page_size, _ = k_cache.shape
+    Hkv, Dv = v_cache.shape[1], v_cache.shape[3]
+    if (k_cache.shape[3] != Dk or v_cache.shape[0] != pages or v_cache.shape[2] != page_size
+            or maps <= 0 or Hk != Hkv * maps or Hq % maps or (Hq // maps) % Hkv):
+        raise KernelError(f"attention: q {tuple(q.shape)}, keys {tuple(k_cache.shape)} and values "
+                          f"{tuple(v_cache.shape)} do not fit each other with {maps} maps a head")
+    if out.shape != (T, Hq, Dv) or not out.is_contiguous() or not q.is_contiguous():
+        raise KernelError(f"attention: q and out [{T}, {Hq}, {Dv}] must be contiguous")
+    if max(Dk, Dv) > 640:
+        raise KernelError(f"attention: head sizes {Dk}, {Dv} exceed the kernel's limit of 640")
+    if not (q.dtype == k_cache.dtype == v_cache.dtype) or out.dtype not in (q.dtype, torch.float32):
+        raise KernelError("attention: q and the caches must share one dtype; out has it, or float32")
+    if not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("attention: caches must be contiguous")
+    for name, t in (("q_start", q_start), ("ctx_len", ctx_len), ("work_seq", work_seq),
+                    ("work_qoff", work_qoff)):
+        _i32(t, name)
+    n = ctx_len.numel()
+    if q_start.numel() != n + 1 or work_seq.numel() != work_qoff.numel():
+        raise KernelError("attention: inconsistent sequence tables")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.shape[0] < n \
+            or block_table.stride(1) != 1:
+        raise KernelError("attention: block_table must be int32 [n, max_pages]")
+    _check(library.load("attention").ptl_attention_generic_kv(
+        _ptr(out), ctypes.c_long(out.stride(0)), int(out.dtype == torch.float32 and q.dtype != torch.float32),
+        _ptr(q), ctypes.c_long(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len),
+        _ptr(block_table), int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff),
+        int(work_seq.numel()), Hq, Hkv, int(maps), Dk, Dv, page_size, int(window), ctypes.c_float(scale),
+        _dtype_code(q), _stream()), "attention")
+
+
+# ---------------------------------------------------------------------------
+# Normed queries and keys, results normed head by head (csrc/prepare.hip)
+NORM_NONE, NORM_HEAD, NORM_WHOLE = 0, 1, 2
+GATE_NONE, GATE_SIGMOID, GATE_SILU = 0, 1, 2
+
+
+def _f32_vec(t: Optional[torch.Tensor], n: int, what: str) -> None:
+    if t is not None and (not t.is_cuda or t.dtype != torch.float32 or t.numel() != n or not t.is_contiguous()):
+        raise KernelError(f"{what} must be a contiguous float32 GPU tensor of {n} numbers")
+
+
+def _f32_rows(p: torch.Tensor, what: str) -> None:
+    if not p.is_cuda or p.dim() != 2 or p.dtype != torch.float32 or p.stride(1) != 1:
+        raise KernelError(f"{what} must be a float32 [T, columns] GPU matrix with dense rows")
+
+
+def qkv_prepare(q_out: torch.Tensor, p: torch.Tensor, q_off: int, k_off: int, v_off: int,
+                q_bias, k_bias, v_bias, norm_mode: int, q_weight, k_weight, eps: float,
+                rot_dims: int, inv_freq, mag: float, positions: torch.Tensor, slots, k_cache, v_cache,
+                Hq: int, Hk: int, Hv: int, Dk: int, Dv: int, page_size: int) -> None:
+    """Bias, norm of queries and keys, rotation and cache write for one step (csrc/prepare.hip).
+    p float32 [T, columns] holds q (Hq heads of Dk) at q_off, k (Hk of Dk) at k_off and v (Hv of
+    Dv) at v_off; k_off < 0: the layer has no keys and values of its own. q_out [T, Hq, Dk] and
+    the caches (k [pages, Hk, page_size, Dk], v [pages, Hv, page_size, Dv]) share one dtype."""
+    _f32_rows(p, "qkv_prepare: p")
+    T = p.shape[0]
+    own = k_off >= 0
+    nq, nk, nv = Hq * Dk, Hk * Dk, Hv * Dv
+    if q_off < 0 or q_off + nq > p.shape[1] or (own and (k_off + nk > p.shape[1] or v_off < 0
+                                                         or v_off + nv > p.shape[1])):
+        raise KernelError("qkv_prepare: the columns of q, k or v lie outside p")
+    if q_out.shape != (T, Hq, Dk) or not q_out.is_contiguous() or not q_out.is_cuda:
+        raise KernelError(f"qkv_prepare: q_out must be a contiguous [{T}, {Hq}, {Dk}] GPU tensor")
+    _f32_vec(q_bias, nq, "qkv_prepare: q bias")
+    nw_q, nw_k = (nq, nk) if norm_mode == NORM_WHOLE else (Dk, Dk)
+    if norm_mode != NORM_NONE:
+        if q_weight is None or (own and k_weight is None):
+            raise KernelError("qkv_prepare: a norm needs its weights")
+        _f32_vec(q_weight, nw_q, "qkv_prepare: q norm weight")
+    if rot_dims:
+        if rot_dims % 2 or rot_dims > Dk:
+            raise KernelError(f"qkv_prepare: {rot_dims} rotating entries of {Dk}")
+        _f32_vec(inv_freq, rot_dims // 2, "qkv_prepare: frequencies")
+    _i32(positions, "positions")
+    if positions.numel() != T:
+        raise KernelError("qkv_prepare: one position a row")
+    write = own and slots is not None
+    if own:
+        _f32_vec(k_bias, nk, "qkv_prepare: k bias")
+        _f32_vec(v_bias, nv, "qkv_prepare: v bias")
+        if norm_mode != NORM_NONE:
+            _f32_vec(k_weight, nw_k, "qkv_prepare: k norm weight")
+    if write:
+        _i32(slots, "slots")
+        _need_gpu(k_cache, v_cache, slots)
+        if (slots.numel() != T or k_cache.dim() != 4 or v_cache.dim() != 4
+                or k_cache.shape[1:] != (Hk, page_size, Dk) or v_cache.shape[1:] != (Hv, page_size, Dv)
+                or k_cache.shape[0] != v_cache.shape[0] or k_cache.dtype != q_out.dtype
+                or v_cache.dtype != q_out.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+            raise KernelError("qkv_prepare: caches must be contiguous [pages, heads, page_size, size] of "
+                              "q_out's dtype, with one slot a row")
+    _check(library.load("prepare").ptl_qkv_prepare(
+        _ptr(q_out), _ptr(p), ctypes.c_long(p.stride(0)), int(q_off), int(k_off) if own else -1, int(v_off),
+        _ptr(q_bias), _ptr(k_bias) if own else None, _ptr(v_bias) if own else None, int(norm_mode),
+        _ptr(q_weight), _ptr(k_weight) if own else None, ctypes.c_float(eps), int(rot_dims),
+        _ptr(inv_freq) if rot_dims else None, ctypes.c_float(mag), _ptr(positions),
+        _ptr(slots) if write else None, _ptr(k_cache) if write else None, _ptr(v_cache) if write else None,
+        T, Hq, Hk, Hv, Dk, Dv, int(page_size), _dtype_code(q_out), _stream()), "qkv_prepare")
+
+
+def head_norm_gate(out: torch.Tensor, a: torch.Tensor, maps: int = 1, lam: float = 0.0, weight=None,
+                   weight_per_head: bool = False, mult: float = 1.0, gate: Optional[torch.Tensor] = None,
+                   gate_off: int = 0, act: int = GATE_NONE, eps: float = 0.0) -> None:
+    """out[t, h, :] = rmsnorm(o)(no weight) * weight * mult * act(gate[t, gate_off + h Dv + :]) with
+    o = a[t, h] (maps 1) or a[t, 2h] - lam a[t, 2h + 1] (maps 2), a float32 [T, H * maps, Dv]
+    contiguous, out [T, H * Dv] (rows may be strided) float32 or bfloat16, gate a float32 matrix."""
+    _need_gpu(out, a, weight, gate)
+    if a.dim() != 3 or a.dtype != torch.float32 or not a.is_contiguous() or maps not in (1, 2) or a.shape[1] % maps:
+        raise KernelError("head_norm_gate: a must be contiguous float32 [T, H * maps, Dv], maps 1 or 2")
+    T, HA, Dv = a.shape
+    H = HA // maps
+    if out.dim() != 2 or out.shape != (T, H * Dv) or out.stride(1) != 1:
+        raise KernelError(f"head_norm_gate: out must be [{T}, {H * Dv}] with dense rows")
+    if weight is not None:
+        _f32_vec(weight, H * Dv if weight_per_head else Dv, "head_norm_gate: weight")
+    ldg = 0
+    if gate is not None:
+        _f32_rows(gate, "head_norm_gate: gate")
+        if gate.shape[0] != T or gate_off < 0 or gate_off + H * Dv > gate.shape[1] or act == GATE_NONE:
+            raise KernelError("head_norm_gate: the gate's columns lie outside its matrix, or no activation")
+        ldg = gate.stride(0)
+    _check(library.load("prepare").ptl_head_norm_gate(
+        _ptr(out), ctypes.c_long(out.stride(0)), _ptr(a), int(maps), ctypes.c_float(lam), _ptr(weight),
+        Dv if weight_per_head else 0, ctypes.c_float(mult), _ptr(gate), ctypes.c_long(ldg), int(gate_off),
+        int(act), ctypes.c_float(eps), T, H, Dv, _dtype_code(out), _stream()), "head_norm_gate")
+
+
+def stream_add_rmsnorm_sum(stream: torch.Tensor, y1: torch.Tensor, a: float, y2: Optional[torch.Tensor],
+                           b: float, bias: Optional[torch.Tensor], c: float, weight: torch.Tensor,
+                           eps: float, out_dtype: Optional[torch.dtype] = None, want_copy: bool = False):
+    """stream += rmsnorm(a y1 + b y2 + c bias) * weight in place (y2 and bias optional); returns a
+    copy of the new stream in ``out_dtype`` when asked, else None."""
+    T, H = _check_stream(stream, "stream_add_rmsnorm_sum")
+    _need_gpu(y1, y2, bias, weight)
+    for y in (y1, y2):
+        if y is not None and (y.shape != stream.shape or not y.is_contiguous() or y.dtype != y1.dtype):
+            raise KernelError("stream_add_rmsnorm_sum: the terms must be contiguous matrices of the stream's "
+                              "shape and of one dtype")
+    _f32_vec(bias, H, "stream_add_rmsnorm_sum: bias")
+    _f32_vec(weight, H, "stream_add_rmsnorm_sum: weight")
+    out_dtype = out_dtype or torch.float32
+    copy = torch.empty((T, H), dtype=out_dtype, device=stream.device) if want_copy else None
+    _check(library.load("stream").ptl_stream_add_rmsnorm_sum(
+        _ptr(stream), _ptr(y1), ctypes.c_float(a), _ptr(y2), ctypes.c_float(b), _dtype_code(y1), _ptr(bias),
+        ctypes.c_float(c), _ptr(weight), ctypes.c_float(eps), _ptr(copy),
+        _F32 if out_dtype == torch.float32 else _BF16, T, H, _stream()), "stream_add_rmsnorm_sum")
+    return copy
+
+
+def stream_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """rmsnorm(x) * weight for rows x of a float32 stream, in ``out_dtype``."""
+    T, H = _check_stream(x, "stream_rmsnorm")
+    _need_gpu(weight)
+    _f32_vec(weight, H, "stream_rmsnorm: weight")
+    out = torch.empty((T, H), dtype=out_dtype, device=x.device)
+    _check(library.load("stream").ptl_stream_rmsnorm(
+        _ptr(out), _F32 if out_dtype == torch.float32 else _BF16, _ptr(x), _ptr(weight), ctypes.c_float(eps),
+        T, H, _stream()), "stream_rmsnorm")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Matrices carried from token to token (csrc/recurrent.hip)
+def recurrent_block_floats(D: int) -> int:
+    """Floats that 16 columns of a head's matrix take in a state slot (with n and m behind them)."""
+    return 16 * D + D + 4
+
+
+def recurrent_state_floats(H: int, D: int, Dv: int) -> int:
+    """Floats of the matrices of all heads in a state slot."""
+    return H * (-(-Dv // 16)) * recurrent_block_floats(D)
+
+
+def _check_scan(state, q_start, state_slots, H, D, Dv, what):
+    _need_gpu(state, q_start, state_slots)
+    _i32(q_start, "q_start")
+    _i32(state_slots, "state_slots")
+    if state.dim() != 2 or state.dtype != torch.float32 or not state.is_contiguous() \
+            or state.shape[1] < recurrent_state_floats(H, D, Dv):
+        raise KernelError(f"{what}: state must be contiguous float32 [slots, >= {recurrent_state_floats(H, D, Dv)}]")
+    n = state_slots.numel()
+    if q_start.numel() != n + 1:
+        raise KernelError(f"{what}: q_start has one entry more than there are sequences")
+    if D > 256:
+        raise KernelError(f"{what}: key sizes up to 256, got {D}")
+    return n
+
+
+def conv_prepare(p: torch.Tensor, x_off: int, conv_weight: torch.Tensor, state: torch.Tensor, tail_off: int,
+                 q_start: torch.Tensor, state_slots: torch.Tensor, G: int, H: int, D: int, Dv: int,
+                 qscale: float):
+    """Short causal convolutions over time, SiLU, unit norm of q and k (csrc/recurrent.hip). p
+    float32 [T, columns] holds the inputs q | k | v (G heads of D, G of D, H of Dv) from x_off on;
+    conv_weight float32 [C, taps]; the state slots hold the last taps - 1 inputs [taps - 1, C] at
+    tail_off. Returns float32 q [T, G, D] (unit vectors times qscale), k [T, G, D], v [T, H, Dv]."""
+    _f32_rows(p, "conv_prepare: p")
+    T = p.shape[0]
+    C = 2 * G * D + H * Dv
+    n = _check_scan(state, q_start, state_slots, H, D, Dv, "conv_prepare")
+    if conv_weight.dim() != 2 or conv_weight.shape[0] != C:
+        raise KernelError(f"conv_prepare: conv_weight must be [{C}, taps]")
+    taps = conv_weight.shape[1]
+    _f32_vec(conv_weight, C * taps, "conv_prepare: conv_weight")
+    if x_off < 0 or x_off + C > p.shape[1] or tail_off < 0 or tail_off + (taps - 1) * C > state.shape[1]:
+        raise KernelError("conv_prepare: columns outside p, or the tail outside the state")
+    qn = torch.empty((T, G, D), dtype=torch.float32, device=p.device)
+    kn = torch.empty((T, G, D), dtype=torch.float32, device=p.device)
+    vv = torch.empty((T, H, Dv), dtype=torch.float32, device=p.device)
+    _check(library.load("recurrent").ptl_conv_prepare(
+        _ptr(qn), _ptr(kn), _ptr(vv), _ptr(p), ctypes.c_long(p.stride(0)), int(x_off), _ptr(conv_weight),
+        int(taps), _ptr(state), ctypes.c_long(state.stride(0)), ctypes.c_long(tail_off), _ptr(q_start),
+        _ptr(state_slots), n, T, G, H, D, Dv, ctypes.c_float(qscale), _stream()), "conv_prepare")
+    return qn, kn, vv
+
+
+def conv_tail_update(p: torch.Tensor, x_off: int, C: int, taps: int, state: torch.Tensor, tail_off: int,
+                     q_start: torch.Tensor, state_slots: torch.Tensor) -> None:
+    """The slots' last taps - 1 inputs after this step (after conv_prepare has read the old ones)."""
+    _f32_rows(p, "conv_tail_update: p")
+    _need_gpu(state, q_start, state_slots)
+    if state.dim() != 2 or state.dtype != torch.float32 or not state.is_contiguous() \
+            or tail_off + (taps - 1) * C > state.shape[1] or x_off + C > p.shape[1]:
+        raise KernelError("conv_tail_update: the tail lies outside the state, or the inputs outside p")
+    _i32(q_start, "q_start")
+    _i32(state_slots, "state_slots")
+    _check(library.load("recurrent").ptl_conv_tail_update(
+        _ptr(state), ctypes.c_long(state.stride(0)), ctypes.c_long(tail_off), _ptr(p),
+        ctypes.c_long(p.stride(0)), int(x_off), _ptr(q_start), _ptr(state_slots), state_slots.numel(),
+        int(C), int(taps), _stream()), "conv_tail_update")
+
+
+def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, p: torch.Tensor, a_off: int, b_off: int,
+               A_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor,
+               state_slots: torch.Tensor) -> torch.Tensor:
+    """The gated delta rule over the rows of every sequence, from and to the state slots. q, k
+    float32 [T, G, D], v float32 [T, H, Dv]; the raw gates a (decay) and b (beta) are columns
+    a_off + h and b_off + h of the float32 matrix p. Returns float32 [T, H, Dv]."""
+    T, G, D = q.shape
+    H, Dv = v.shape[1], v.shape[2]
+    _f32_rows(p, "delta_scan: p")
+    n = _check_scan(state, q_start, state_slots, H, D, Dv, "delta_scan")
+    for t, shape in ((q, (T, G, D)), (k, (T, G, D)), (v, (T, H, Dv))):
+        if t.shape != shape or t.dtype != torch.float32 or not t.is_contiguous() or not t.is_cuda:
+            raise KernelError("delta_scan: q, k [T, G, D] and v [T, H, Dv] must be contiguous float32")
+    if H % G or min(a_off, b_off) < 0 or max(a_off, b_off) + H > p.shape[1] or p.shape[0] != T:
+        raise KernelError("delta_scan: gates outside p, or heads that do not divide")
+    _f32_vec(A_log, H, "delta_scan: A_log")
+    _f32_vec(dt_bias, H, "delta_scan: dt_bias")
+    out = torch.empty((T, H, Dv), dtype=torch.float32, device=q.device)
+    pa, pb = p[:, a_off:], p[:, b_off:]
+    _check(library.load("recurrent").ptl_delta_scan(
+        _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pa), _ptr(pb), ctypes.c_long(p.stride(0)), _ptr(A_log),
+        _ptr(dt_bias), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(q_start), _ptr(state_slots), n,
+        H, G, D, Dv, _stream()), "delta_scan")
+    return out
+
+
+def memory_scan(p: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: int, f_off: int,
+                i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float, qscale: float, state: torch.Tensor,
+                q_start: torch.Tensor, state_slots: torch.Tensor, H: int, D: int, Dv: int) -> torch.Tensor:
+    """The matrix memory with exponential gates and a running maximum over the rows of every
+    sequence, from and to the state slots. q, k (H heads of D), v (H of Dv) and the raw gates i, f
+    (H each) are columns of the float32 matrix p. Returns float32 [T, H, Dv]."""
+    _f32_rows(p, "memory_scan: p")
+    T = p.shape[0]
+    n = _check_scan(state, q_start, state_slots, H, D, Dv, "memory_scan")
+    for off, width in ((q_off, H * D), (k_off, H * D), (v_off, H * Dv), (i_off, H), (f_off, H)):
+        if off < 0 or off + width > p.shape[1]:
+            raise KernelError("memory_scan: columns outside p")
+    _f32_vec(i_bias, H, "memory_scan: i bias")
+    _f32_vec(f_bias, H, "memory_scan: f bias")
+    out = torch.empty((T, H, Dv), dtype=torch.float32, device=p.device)
+    _check(library.load("recurrent").ptl_memory_scan(
+        _ptr(out), _ptr(p), ctypes.c_long(p.stride(0)), int(q_off), int(k_off), int(v_off), int(i_off),
+        int(f_off), _ptr(i_bias), _ptr(f_bias), ctypes.c_float(cap), ctypes.c_float(qscale), _ptr(state),
+        ctypes.c_long(state.stride(0)), _ptr(q_start), _ptr(state_slots), n, H, D, Dv, _stream()),
+        "memory_scan")
+    return out
+
+
+# ---------------------------------------------------------------------------
 # Routed experts (csrc/moe.hip)
 ACT_SILU, ACT_CLAMPED = 0, 1
 

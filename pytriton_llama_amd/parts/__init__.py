@@ -3,10 +3,12 @@ from .base import (PART_KINDS, PART_REGISTRY, PagedSpec, PagedTensor, ParamSourc
                    place, register_part)
 from .linear import linear
 from .norm import DynamicTanh, RMSNorm
-from .rotary import RotaryEncoding, default_inv_freq, llama3_inv_freq
+from .rotary import RotaryEncoding, default_inv_freq, llama3_inv_freq, ramp_inv_freq
 from .attention import PagedAttention
 from .feedforward import GatedMLP, RoutedExperts, SwiGLU
 from .latent_attention import LatentAttention
 from .token_input import GatedTokenInput, TokenTable
 from .embedding import LinearHead, TokenEmbedding
-from .block import PreNormBlock, SandwichBlock
+from .normed_attention import NormedAttention
+from .recurrent import GatedDeltaRule, MatrixMemory, ParallelMixers
+from .block import OutputNormBlock, PreNormBlock, SandwichBlock

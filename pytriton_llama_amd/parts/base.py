@@ -40,7 +40,10 @@ inside a kernel it launches anyway:
                               norm returns it when called with scale_ok=True; a mixer or
                               feed-forward whose class says ``takes_pending_scale`` applies the
                               factor to the results of its first product.
-Both have .tensor(), which finishes the work with separate kernels. The block (and the model,
+    PendingSum(terms, bias)   a weighted sum of one or two results and a bias, not added up; a
+                              block with a norm on its sublayers' outputs adds it up inside that
+                              norm's kernel.
+All have .tensor(), which finishes the work with separate kernels. The block (and the model,
 between blocks) asks the classes for these flags and passes plain tensors to everyone else.
 
 ``ctx`` is the StepContext of engine/batch.py: the flat batch (positions,
@@ -166,9 +169,34 @@ class PendingScale:
         return ops.row_scale(self.values, self.scale)
 
 
+class PendingSum:
+    """a y1 + b y2 + c bias that has not been added up: what a mixer returns whose result is a
+    weighted sum (two mixers side by side, an output projection with a bias). ``terms``: one or two
+    (matrix [T, hidden], factor); ``bias``: (float32 vector [hidden], factor) or None. A block
+    whose next kernel reads the result anyway (a norm on the sublayer's output) adds it up there."""
+    __slots__ = ("terms", "bias")
+
+    def __init__(self, terms, bias=None):
+        if not 1 <= len(terms) <= 2:
+            raise ValueError("a pending sum has one or two terms")
+        self.terms, self.bias = list(terms), bias
+
+    @property
+    def shape(self):
+        return self.terms[0][0].shape
+
+    def tensor(self) -> torch.Tensor:
+        out = self.terms[0][0].float() * self.terms[0][1]
+        for y, f in self.terms[1:]:
+            out = out + y.float() * f
+        if self.bias is not None:
+            out = out + self.bias[0] * self.bias[1]
+        return out.to(self.terms[0][0].dtype)
+
+
 def as_tensor(v):
     """``v`` finished, if it is one of the pending values."""
-    return v.tensor() if isinstance(v, (PendingProduct, PendingScale)) else v
+    return v.tensor() if isinstance(v, (PendingProduct, PendingScale, PendingSum)) else v
 
 
 def run_norm(norm, x, residual, consumer=None):

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from .. import ops
-from .base import Part, as_tensor, register_part, run_norm
+from .base import Part, PendingSum, as_tensor, register_part, run_norm
 
 
 @register_part("block", "prenorm")
@@ -187,3 +187,82 @@ class SandwichBlock(Part):
                         return self.dtype
             raise RuntimeError("the block's parts hold no weights yet")
         return self.dtype
+
+
+@register_part("block", "output_norm")
+class OutputNormBlock(Part):
+    """A norm on every sublayer's output only, on a residual stream kept in float32:
+
+        x <- x + norm1(mixer(x));   x <- x + norm2(ffn(x))
+
+    The sublayers read x itself (in the engine's dtype); the feed-forward with its norm is
+    optional. The norms are RMS norms: the norm, the sum into the stream and the copy of the new
+    stream in the engine's dtype for the next sublayer are one kernel, which also adds up a
+    sublayer's result that arrives as a weighted sum not yet made (parts.base.PendingSum). The
+    stream is the block's ``h`` (float32 [T, hidden], updated in place); what the block returns
+    where others carry a residual is that copy, and a block that is handed one starts from it.
+    ``last`` (set by the model's builder): nobody reads the copy after this block."""
+
+    def __init__(self, mixer: Part, mixer_norm: Part, feed_forward: Part = None, ffn_norm: Part = None):
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward comes with its norm, or neither")
+        for n in (mixer_norm, ffn_norm):
+            if n is not None and not (hasattr(n, "weight") and hasattr(n, "eps")):
+                raise ValueError("the norms of this block are RMS norms (a weight and an eps)")
+        self.mixer, self.norm1 = mixer, mixer_norm
+        self.feed_forward, self.norm2 = feed_forward, ffn_norm
+        libs = ("stream",)
+        for p in self.children().values():
+            libs += tuple(p.kernel_libraries)
+        self.kernel_libraries = tuple(dict.fromkeys(libs))
+        self.last = False
+
+    def children(self):
+        roles = {"mixer": self.mixer, "norm1": self.norm1, "feed_forward": self.feed_forward,
+                 "norm2": self.norm2}
+        return {k: p for k, p in roles.items() if p is not None}
+
+    def cache_spec(self):
+        return self.mixer.cache_spec() if hasattr(self.mixer, "cache_spec") else None
+
+    def work_lists(self):
+        lists = ()
+        for p in self.children().values():
+            if hasattr(p, "work_lists"):
+                lists += tuple(p.work_lists())
+        return tuple(dict.fromkeys(lists))
+
+    def make_decode_copies(self) -> int:
+        return sum(p.make_decode_copies() for p in self.children().values()
+                   if hasattr(p, "make_decode_copies"))
+
+    @property
+    def graph_capturable(self) -> bool:
+        return all(getattr(p, "graph_capturable", True) for p in self.children().values())
+
+    @staticmethod
+    def _add(stream, y, norm, dtype, want_copy):
+        """stream += norm(y); returns the new stream in ``dtype`` when asked (the stream itself
+        when that is float32)."""
+        copy = want_copy and dtype != torch.float32
+        if isinstance(y, PendingSum):
+            (y1, a), (y2, b) = y.terms[0], (y.terms[1] if len(y.terms) > 1 else (None, 0.0))
+            bias, c = y.bias if y.bias is not None else (None, 0.0)
+            out = ops.stream_add_rmsnorm_sum(stream, y1, a, y2, b, bias, c, norm.weight, norm.eps, dtype, copy)
+        else:
+            _, out = ops.stream_add_rmsnorm(stream, as_tensor(y), norm.weight, norm.eps, None, dtype, copy)
+        return out if copy else (stream if want_copy else None)
+
+    def forward(self, h, residual, ctx, cache):
+        if h.dtype != torch.float32:
+            raise ops.KernelError("an output-norm block runs on a float32 residual stream")
+        stream, dtype = h, self.norm1.dtype
+        a = residual
+        if a is None:
+            a = stream if dtype == torch.float32 else ops.stream_add_dyt(stream, None, None, None, dtype, True)[1]
+        y = self.mixer.forward(a, ctx, cache)
+        if self.feed_forward is None:
+            return stream, self._add(stream, y, self.norm1, dtype, not self.last)
+        a = self._add(stream, y, self.norm1, dtype, True)
+        y = self.feed_forward.forward(a)
+        return stream, self._add(stream, y, self.norm2, dtype, not self.last)

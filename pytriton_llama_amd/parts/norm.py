@@ -15,7 +15,7 @@ class RMSNorm(Part):
     sum returned as the new residual (lite_llama/kernels/skip_rmsnorm.py:94-181;
     call sites lite_llama/models/llama.py:149,160,219). Without a residual the
     input itself is the residual (:181)."""
-    kernel_libraries = ("norm", "gemm", "gemm_rows")
+    kernel_libraries = ("norm", "gemm", "gemm_rows", "stream")
     takes_pending_product = True
 
     def __init__(self, size: int, eps: float, weight_name: str = "weight"):
@@ -23,12 +23,14 @@ class RMSNorm(Part):
         self.eps = float(eps)
         self.weight_name = weight_name
         self.weight: Optional[torch.Tensor] = None
+        self.dtype: Optional[torch.dtype] = None
 
     def param_sources(self) -> List[ParamSource]:
         return [ParamSource(self.weight_name, (self.size,), "vector")]
 
     def load(self, tensors, dtype, device) -> None:
         self.weight = place(tensors[self.weight_name], "vector", dtype, device)
+        self.dtype = dtype
 
     def forward(self, x, residual: Optional[torch.Tensor], scale_ok: bool = False):
         if isinstance(x, PendingProduct):
@@ -46,6 +48,9 @@ class RMSNorm(Part):
                                                     blocked=x.blocked)
                 return PendingScale(y, scale), residual
         x = as_tensor(x)
+        if residual is None and x.dtype == torch.float32 and self.dtype not in (None, torch.float32):
+            # rows of a residual stream that is kept in float32: the result in the engine's dtype
+            return ops.stream_rmsnorm(x, self.weight, self.eps, self.dtype), x
         y = ops.add_rmsnorm(x, residual, self.weight, self.eps)
         return y, (x if residual is None else residual)
 

@@ -33,6 +33,25 @@ def llama3_inv_freq(theta: float, dim: int, factor: float, low_freq_factor: floa
     return torch.where(medium, blended, scaled)
 
 
+def ramp_inv_freq(base: float, dims: int, factor: float, original: float, fast: float, slow: float):
+    """Frequencies that go over from the unscaled f_i = base^(-2i/dims) (fast entries) to f_i /
+    factor (slow entries) along a linear ramp, and the factor on sine and cosine that goes with
+    them (the "YaRN" scaling of Peng, Quesnelle, Fan and Shippole). The ramp runs between the
+    entries that make ``fast`` and ``slow`` turns over ``original`` positions:
+    e(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(e(fast)), 0), hi =
+    min(ceil(e(slow)), dims - 1), ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1).
+    Returns (float32 [dims / 2], 0.1 ln(factor) + 1); worked out in float64, rounded once."""
+    i = torch.arange(0, dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+
+    def entry(turns: float) -> float:
+        return dims * math.log(original / (2 * math.pi * turns)) / (2 * math.log(base))
+    lo = max(math.floor(entry(fast)), 0)
+    hi = min(math.ceil(entry(slow)), dims - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return (f / factor * ramp + f * (1.0 - ramp)).to(torch.float32), 0.1 * math.log(factor) + 1.0
+
+
 @register_part("position", "rotary")
 class RotaryEncoding(Part):
     """Rotate-half RoPE. ``rope_type`` "default" or "llama3" with its four numbers
