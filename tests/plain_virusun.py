@@ -12,6 +12,27 @@ import math
 import torch
 
 
+# The dtype an engine rounds to where it stores a result between kernels (keys and values in the
+# cache, queries, the heads' results in front of an output projection, a feed-forward's hidden
+# values and result); None: nothing is rounded. Set by forward(round_inputs=...).
+ROUND_TO = None
+
+
+# When a list: every recurrent mixer appends a tensor [T] to it, the smallest ratio over its heads of
+# |S^T q| to | |S|^T |q| | at each position: how much of the read-out is left after cancellation. The
+# norm that follows keeps the direction of the read-out and drops its size, so where the ratio is
+# small the direction (behind a single token: the sign of k . q) is decided by rounding.
+CANCELLATION = None
+
+
+def _left_of_readout(S, q, o):
+    return (o.norm() / ((S.abs().T @ q.abs()).norm() + 1e-30)).item()
+
+
+def stored(x):
+    return x if ROUND_TO is None else x.to(ROUND_TO).to(x.dtype)
+
+
 def rms(x, eps):
     """x / sqrt(mean(x^2) + eps) over the last axis."""
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
@@ -70,7 +91,7 @@ def diff_keys_values(h, m, t, pre, eps):
     k = lin(h, t[pre + "k"], t[pre + "k.b"]).view(T, G, 2, D)
     k = rms(k, eps) * t[pre + "k.norm"]
     v = lin(h, t[pre + "v"], t[pre + "v.b"]).view(T, G, Dv)
-    return k, v
+    return stored(k), stored(v)
 
 
 def differential_attention(h, m, t, pre, eps, kv):
@@ -78,7 +99,7 @@ def differential_attention(h, m, t, pre, eps, kv):
     T = h.shape[0]
     H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = lin(h, t[pre + "q"], t[pre + "q.b"]).view(T, H, 2, D)
-    q = rms(q, eps) * t[pre + "q.norm"]
+    q = stored(rms(q, eps) * t[pre + "q.norm"])
     k, v = kv
     rep = H // G
     k = k.repeat_interleave(rep, dim=1)                     # [T, H, 2, D]
@@ -91,7 +112,7 @@ def differential_attention(h, m, t, pre, eps, kv):
     o = a[:, :, 0] - lam * a[:, :, 1]
     o = rms(o, eps) * (1.0 - m["diff"])
     o = o.reshape(T, H * Dv) * torch.sigmoid(lin(h, t[pre + "g"]))
-    return lin(o, t[pre + "o"], t[pre + "o.b"])
+    return lin(stored(o), t[pre + "o"], t[pre + "o.b"])
 
 
 def rotary_attention(h, m, t, pre, eps):
@@ -100,12 +121,12 @@ def rotary_attention(h, m, t, pre, eps):
     pos = torch.arange(T)
     q = rms(lin(h, t[pre + "q"], t[pre + "q.b"]), eps) * t[pre + "q.norm"]
     k = rms(lin(h, t[pre + "k"], t[pre + "k.b"]), eps) * t[pre + "k.norm"]
-    q = rotate_half(q.view(T, H, D), pos, m["rot"])
-    k = rotate_half(k.view(T, G, D), pos, m["rot"]).repeat_interleave(H // G, dim=1)
-    v = lin(h, t[pre + "v"], t[pre + "v.b"]).view(T, G, Dv).repeat_interleave(H // G, dim=1)
+    q = stored(rotate_half(q.view(T, H, D), pos, m["rot"]))
+    k = stored(rotate_half(k.view(T, G, D), pos, m["rot"])).repeat_interleave(H // G, dim=1)
+    v = stored(lin(h, t[pre + "v"], t[pre + "v.b"])).view(T, G, Dv).repeat_interleave(H // G, dim=1)
     p = causal_softmax(torch.einsum("ihd,jhd->hij", q, k) * m["scale"])
     o = torch.einsum("hij,jhe->ihe", p, v).reshape(T, H * Dv)
-    return lin(o, t[pre + "o"], t[pre + "o.b"])
+    return lin(stored(o), t[pre + "o"], t[pre + "o.b"])
 
 
 def matrix_memory(h, m, t, pre, eps):
@@ -118,6 +139,7 @@ def matrix_memory(h, m, t, pre, eps):
     gi = cap * torch.tanh(lin(h, t[pre + "i"], t[pre + "i.b"]) / cap)                     # [T, H]
     gf = torch.nn.functional.logsigmoid(cap * torch.tanh(lin(h, t[pre + "f"], t[pre + "f.b"]) / cap))
     out = torch.zeros(T, H, Dv, dtype=h.dtype)
+    left = torch.ones(T)
     for hd in range(H):
         S = torch.zeros(D, Dv, dtype=h.dtype)
         n = torch.zeros(D, dtype=h.dtype)
@@ -130,8 +152,11 @@ def matrix_memory(h, m, t, pre, eps):
             mx = m_new
             den = torch.maximum((n @ q[s, hd]).abs(), torch.exp(-mx)) + 1e-6
             out[s, hd] = (S.T @ q[s, hd]) / den
+            left[s] = min(left[s], _left_of_readout(S, q[s, hd], S.T @ q[s, hd]))
+    if CANCELLATION is not None:
+        CANCELLATION.append(left)
     o = rms(out, eps).reshape(T, H * Dv) * t[pre + "norm"] * torch.sigmoid(lin(h, t[pre + "g"]))
-    return lin(o, t[pre + "o"])
+    return lin(stored(o), t[pre + "o"])
 
 
 def short_conv(x, w):
@@ -154,6 +179,7 @@ def gated_delta(h, m, t, pre, eps):
     decay = torch.exp(-torch.exp(t[pre + "A_log"]) * torch.nn.functional.softplus(
         lin(h, t[pre + "a"]) + t[pre + "dt_bias"]))
     out = torch.zeros(T, H, Dv, dtype=h.dtype)
+    left = torch.ones(T)
     for hd in range(H):
         g = hd // (H // G)
         S = torch.zeros(D, Dv, dtype=h.dtype)
@@ -162,18 +188,37 @@ def gated_delta(h, m, t, pre, eps):
             u = beta[s, hd] * (v[s, hd] - S.T @ k[s, g])
             S = S + torch.outer(k[s, g], u)
             out[s, hd] = S.T @ q[s, g]
+            left[s] = min(left[s], _left_of_readout(S, q[s, g], out[s, hd]))
+    if CANCELLATION is not None:
+        CANCELLATION.append(left)
     o = rms(out, eps) * t[pre + "norm"]
     o = o.reshape(T, H * Dv) * silu(lin(h, t[pre + "g"]))
-    return lin(o, t[pre + "o"])
+    return lin(stored(o), t[pre + "o"])
 
 
 def dense_ff(h, t, pre):
-    return lin(silu(lin(h, t[pre + "gate"])) * lin(h, t[pre + "up"]), t[pre + "down"])
+    return stored(lin(stored(silu(lin(h, t[pre + "gate"])) * lin(h, t[pre + "up"])), t[pre + "down"]))
 
 
 # ---- the model ---------------------------------------------------------------------------------
-def forward(config, tensors, tokens, dtype=torch.float64, return_layers=False):
-    """Logits [T, vocab] of one whole sequence (and the stream after every layer)."""
+def forward(config, tensors, tokens, dtype=torch.float64, return_layers=False, round_inputs=None,
+            cancellation_out=None):
+    """Logits [T, vocab] of one whole sequence (and the stream after every layer).
+    ``round_inputs``: a dtype that every sublayer's input, and what an engine stores between
+    kernels (see ROUND_TO), is rounded to, as an engine of that dtype rounds it (the stream itself
+    is not rounded). ``cancellation_out``: a list that receives one tensor [T] a recurrent mixer (see
+    CANCELLATION)."""
+    global ROUND_TO, CANCELLATION
+    ROUND_TO, CANCELLATION = round_inputs, cancellation_out
+    try:
+        return _forward(config, tensors, tokens, dtype, return_layers)
+    finally:
+        ROUND_TO = CANCELLATION = None
+
+
+def _forward(config, tensors, tokens, dtype, return_layers):
+    seen = stored
+
     t = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in tensors.items()}
     eps = float(config["norm"]["eps"])
     x = t["embed"][torch.as_tensor(tokens, dtype=torch.long)]
@@ -184,18 +229,18 @@ def forward(config, tensors, tokens, dtype=torch.float64, return_layers=False):
         if kind == "attention":
             src = m.get("kv_from")
             if src is None:
-                kept[i] = diff_keys_values(x, m, t, pre, eps)
-            y = differential_attention(x, m, t, pre, eps, kept[i if src is None else src])
+                kept[i] = diff_keys_values(seen(x), m, t, pre, eps)
+            y = differential_attention(seen(x), m, t, pre, eps, kept[i if src is None else src])
         elif kind == "parallel":
-            y = (m["left_scale"] * rotary_attention(x, m["left"], t, pre + "left.", eps)
-                 + m["right_scale"] * matrix_memory(x, m["right"], t, pre + "right.", eps))
+            y = (m["left_scale"] * rotary_attention(seen(x), m["left"], t, pre + "left.", eps)
+                 + m["right_scale"] * matrix_memory(seen(x), m["right"], t, pre + "right.", eps))
         elif kind == "delta":
-            y = gated_delta(x, m, t, pre, eps)
+            y = gated_delta(seen(x), m, t, pre, eps)
         else:
             raise ValueError(kind)
         x = x + rms(y, eps) * t[f"l{i}.norm1"]
         if layer.get("mlp") is not None:
-            x = x + rms(dense_ff(x, t, f"l{i}.mlp."), eps) * t[f"l{i}.norm2"]
+            x = x + rms(dense_ff(seen(x), t, f"l{i}.mlp."), eps) * t[f"l{i}.norm2"]
         after.append(x)
-    logits = lin(rms(x, eps) * t["final.norm"], t["head"])
+    logits = lin(seen(rms(x, eps) * t["final.norm"]), t["head"])
     return (logits, torch.stack(after)) if return_layers else logits
