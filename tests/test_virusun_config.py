@@ -1,0 +1,116 @@
+"""Virusun's configuration, builder and frequencies on the CPU."""
+import copy
+import math
+
+import pytest
+import torch
+
+import plain_virusun
+from virusun_configs import VIRUSUN, virusun
+
+
+def test_config_reads_every_size_and_constant():
+    from pytriton_llama_amd.config import VirusunConfig
+    cfg, _, _ = virusun("V1")
+    c = VirusunConfig.from_dict(cfg)
+    assert (c.vocab_size, c.hidden_size, c.norm_eps, len(c.layers)) == (200, 64, 1e-5, 5)
+    assert [l.kind for l in c.layers] == ["attention", "delta", "attention", "parallel", "attention"]
+    assert [l.ff for l in c.layers] == [96, 80, 0, 72, 64]
+    a, d, p = c.layers[0].mixer, c.layers[1].mixer, c.layers[3].mixer
+    assert (a.heads, a.kv_heads, a.dim, a.vdim, a.scale, a.diff, a.kv_from) == (6, 2, 16, 24, 0.3, 0.4, None)
+    assert c.layers[2].mixer.kv_from == 0
+    assert (d.heads, d.kv_heads, d.dim, d.vdim, d.conv) == (4, 2, 16, 24, 4)
+    assert (p.left.rot.dims, p.left.rot.base, p.left.rot.scaling) == (32, 10000.0, (4.0, 64.0, 8.0, 1.0))
+    assert (p.right.heads, p.right.gate_cap, p.left_scale, p.right_scale) == (3, 10.0, 0.8, 1.3)
+    assert c.to_dict() == cfg
+
+
+@pytest.mark.parametrize("change,text", [
+    (lambda c: c["layers"][0].update(type="window"), "unknown layer type"),
+    (lambda c: c["layers"][0]["mixer"].pop("diff"), "lacks 'diff'"),
+    (lambda c: c["layers"][2]["mixer"].update(kv_from=1), "no keys and values"),
+    (lambda c: c["layers"][2]["mixer"].update(kv_from=2), "earlier layer"),
+    (lambda c: c["layers"][2]["mixer"].update(vdim=8), "differ from layer 0"),
+    (lambda c: c["layers"][0]["mixer"].update(heads=5), "not a multiple"),
+    (lambda c: c["layers"][3]["mixer"]["left"]["rot"].update(dims=34), "dims 34"),
+    (lambda c: c["layers"][3]["mixer"]["left"]["rot"]["scaling"].pop("slow"), "lacks 'slow'"),
+    (lambda c: c["layers"][3]["mixer"]["right"].update(gate_cap=0), "gate_cap must be positive"),
+    (lambda c: c["layers"][1]["mixer"].update(conv=0), "conv must be positive"),
+    (lambda c: c["layers"][1]["mlp"].update(kind="moe"), "unknown feed-forward kind"),
+    (lambda c: c.pop("norm"), "lacks 'norm'"),
+    (lambda c: c.update(layers=[]), "empty"),
+])
+def test_config_errors_name_the_place(change, text):
+    from pytriton_llama_amd.config import ConfigError, VirusunConfig
+    cfg, _, _ = virusun("V1")
+    change(cfg)
+    with pytest.raises(ConfigError) as e:
+        VirusunConfig.from_dict(cfg)
+    assert text in str(e.value)
+
+
+@pytest.mark.parametrize("name", sorted(VIRUSUN))
+def test_builder_wires_caches_and_names(name):
+    import pytriton_llama_amd  # noqa: F401
+    from pytriton_llama_amd.config import build_model
+    from pytriton_llama_amd.parts import PagedSpec, StateSpec
+    cfg, _, _ = virusun(name)
+    model = build_model(cfg)
+    assert [c.block for c in model.schedule] == list(range(len(cfg["layers"])))
+    owners = {}
+    for i, (layer, call) in enumerate(zip(cfg["layers"], model.schedule)):
+        m = layer["mixer"]
+        if layer["type"] == "attention" and m.get("kv_from") is not None:
+            assert call.cache_layer == owners[m["kv_from"]] and not call.writes
+        elif layer["type"] == "parallel":
+            left, right = call.cache_layer
+            assert isinstance(model.cache_layers[left], PagedSpec) and isinstance(model.cache_layers[right], StateSpec)
+            assert model.cache_layers[right].dtype == torch.float32
+        elif layer["type"] == "delta":
+            assert isinstance(model.cache_layers[call.cache_layer], StateSpec) and call.writes
+        else:
+            owners[i] = call.cache_layer
+            spec = model.cache_layers[call.cache_layer]
+            assert [t.shape for t in spec.tensors] == [(2 * m["kv_heads"], m["dim"]), (m["kv_heads"], m["vdim"])]
+    names = model.expected_tensors()
+    for i, layer in enumerate(cfg["layers"]):
+        m = layer["mixer"]
+        assert names[f"l{i}.norm1"][1].shape == (cfg["width"],)
+        assert (f"l{i}.mlp.down" in names) == (layer["mlp"] is not None) == (f"l{i}.norm2" in names)
+        if layer["type"] == "attention":
+            assert names[f"l{i}.mix.q"][1].shape == (m["heads"] * 2 * m["dim"], cfg["width"])
+            assert (f"l{i}.mix.k" in names) == (m.get("kv_from") is None) == (f"l{i}.mix.k.norm" in names)
+            assert names[f"l{i}.mix.lq1"][1].shape == (m["dim"],)
+        elif layer["type"] == "parallel":
+            assert names[f"l{i}.mix.left.q.norm"][1].shape == (m["left"]["heads"] * m["left"]["dim"],)
+            assert names[f"l{i}.mix.right.i.b"][1].shape == (m["right"]["heads"],)
+            assert names[f"l{i}.mix.right.norm"][1].shape == (m["right"]["heads"] * m["right"]["vdim"],)
+        else:
+            assert names[f"l{i}.mix.v.conv"][1].shape == (m["heads"] * m["vdim"], m["conv"])
+            assert names[f"l{i}.mix.norm"][1].shape == (m["vdim"],)
+    assert {"embed", "head", "final.norm"} <= set(names)
+
+
+def test_random_model_folder_round_trip(tmp_path):
+    from safetensors.torch import load_file
+    from pytriton_llama_amd.config import build_model, read_config_json
+    from pytriton_llama_amd.weights import load_weights, write_random_model
+    cfg, std, _ = virusun("V2")
+    write_random_model(cfg, str(tmp_path), seed=1, dtype=torch.float32, norm_std=0.1, std=std)
+    model = build_model(read_config_json(str(tmp_path)))
+    load_weights(model, str(tmp_path), torch.float32, "cpu")
+    w = load_file(str(tmp_path / "model.safetensors"))
+    assert set(w) == set(model.expected_tensors())
+    logits = plain_virusun.forward(cfg, w, [1, 2, 3, 4, 5])
+    assert logits.shape == (5, cfg["vocab"]) and bool(torch.isfinite(logits).all())
+
+
+@pytest.mark.parametrize("dims,base,scaling", [(64, 10000.0, (4.0, 2048, 32.0, 1.0)), (12, 500.0, (2.0, 32, 4.0, 0.5)),
+                                               (32, 10000.0, (8.0, 128, 16.0, 2.0)), (8, 50.0, (1.5, 16, 3.0, 3.0))])
+def test_ramp_frequencies(dims, base, scaling):
+    from pytriton_llama_amd.parts import ramp_inv_freq
+    got, mag = ramp_inv_freq(base, dims, *scaling)
+    want, wmag = plain_virusun.ramp_frequencies(dims, base, dict(zip(("factor", "original", "fast", "slow"), scaling)))
+    assert torch.equal(got, want.float()) and mag == wmag == 0.1 * math.log(scaling[0]) + 1
+    f = base ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64) / dims)
+    assert bool((got.double() <= f * (1 + 1e-6)).all()) and bool((got.double() >= f / scaling[0] * (1 - 1e-6)).all())
