@@ -236,6 +236,48 @@ RUBASUN_SIZES = {
 }
 
 
+def virusun_shape(width, layers, heads, kv_heads, dim, vdim, memory_heads, delta_heads, delta_kv_heads, ff, vocab):
+    """A Virusun config.json of a real model's layer sizes, four kinds of layers in turn:
+    differential attention with keys and values of its own, rotary attention beside a matrix
+    memory, differential attention that reads the keys and values two layers back, the gated delta
+    rule; a dense feed-forward in each."""
+    diff = {"heads": heads, "kv_heads": kv_heads, "dim": dim // 2, "vdim": vdim, "scale": (dim // 2) ** -0.5,
+            "diff": 0.6}
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+            "rot": {"base": 10000.0, "dims": dim // 2,
+                    "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+    right = {"heads": memory_heads, "dim": dim, "vdim": vdim, "gate_cap": 15.0}
+    delta = {"heads": delta_heads, "kv_heads": delta_kv_heads, "dim": dim, "vdim": vdim, "conv": 4}
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            layer = {"type": "attention", "mixer": dict(diff)}
+        elif kind == 1:
+            layer = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}}
+        elif kind == 2:
+            layer = {"type": "attention", "mixer": dict(diff, kv_from=i - 2)}
+        else:
+            layer = {"type": "delta", "mixer": delta}
+        layer["mlp"] = {"kind": "dense", "ff": ff}
+        out.append(layer)
+    return {"architecture": "Virusun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": out,
+            "initializer_range": 0.02}
+
+
+# name -> (Virusun sizes, the Llama shape of equal width, depth, heads and feed-forward width)
+VIRUSUN_SIZES = {
+    "2048": (dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, vdim=128, memory_heads=8, delta_heads=16,
+                  delta_kv_heads=8, ff=8192, vocab=32000),
+             dict(num_hidden_layers=8, hidden_size=2048, num_attention_heads=16, num_key_value_heads=4,
+                  head_dim=128, intermediate_size=8192, vocab_size=32000, tie_word_embeddings=False)),
+    "4096": (dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, vdim=128, memory_heads=16, delta_heads=32,
+                  delta_kv_heads=16, ff=14336, vocab=32000),
+             dict(num_hidden_layers=4, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                  head_dim=128, intermediate_size=14336, vocab_size=32000, tie_word_embeddings=False)),
+}
+
+
 def engine_rates(cfg, dtype, S, batch, steps, warmup):
     """Prefill of one S-token prompt (one step) and decode steps of ``batch`` requests behind
     S-token prompts, through the whole engine, for any architecture."""
@@ -291,32 +333,40 @@ def _tensors_of(model):
     return [torch.empty(src.shape, device="meta") for _, src in model.expected_tensors().values()]
 
 
-def rubasun_beside_llama(args):
-    """Prefill and decode throughput of Rubasun at layer sizes of real models, beside the
+def beside_llama(args, design, wanted, models, sizes_table, shape):
+    """Prefill and decode throughput of another design at layer sizes of real models, beside the
     Llama decoder of equal width, depth and feed-forward width a token, same engine, same
     measurement. One JSON line."""
     rows = {}
-    for name in [n for n in args.rubasun.split(",") if n]:
-        if name not in RUBASUN_SIZES:
-            print(f"--rubasun takes {sorted(RUBASUN_SIZES)}", file=sys.stderr)
+    for name in [n for n in wanted.split(",") if n]:
+        if name not in sizes_table:
+            print(f"--{design} takes {sorted(sizes_table)}", file=sys.stderr)
             return 2
-        r_sizes, l_shape = RUBASUN_SIZES[name]
+        d_sizes, l_shape = sizes_table[name]
         llama = dict(LLAMA_1B)
         llama.update(l_shape)
-        for label, cfg in (("rubasun", rubasun_shape(**r_sizes)), ("llama", llama)):
-            if label not in args.rubasun_models.split(","):
+        for label, cfg in ((design, shape(**d_sizes)), ("llama", llama)):
+            if label not in models.split(","):
                 continue
             log(f"width {name}: {label}")
             rows[f"{label}_{name}"] = engine_rates(cfg, args.dtype, args.prompt_len, args.batch, args.steps,
                                                    args.warmup)
             log(json.dumps(rows[f"{label}_{name}"]))
-    print(json.dumps({"metric": f"Rubasun beside Llama: prefill of {args.prompt_len} tokens and decode at batch "
-                                f"{args.batch} behind {args.prompt_len}-token prompts",
+    print(json.dumps({"metric": f"{design.capitalize()} beside Llama: prefill of {args.prompt_len} tokens and decode "
+                                f"at batch {args.batch} behind {args.prompt_len}-token prompts",
                       "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                       "data": "synthetic", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-                      "sizes": {n: {"rubasun": RUBASUN_SIZES[n][0], "llama": RUBASUN_SIZES[n][1]}
-                                for n in args.rubasun.split(",") if n}, "rows": rows}), flush=True)
+                      "sizes": {n: {design: sizes_table[n][0], "llama": sizes_table[n][1]}
+                                for n in wanted.split(",") if n}, "rows": rows}), flush=True)
     return 0
+
+
+def rubasun_beside_llama(args):
+    return beside_llama(args, "rubasun", args.rubasun, args.rubasun_models, RUBASUN_SIZES, rubasun_shape)
+
+
+def virusun_beside_llama(args):
+    return beside_llama(args, "virusun", args.virusun, args.virusun_models, VIRUSUN_SIZES, virusun_shape)
 
 
 def main():
@@ -354,6 +404,10 @@ def main():
                          "steps at --batch, both through the whole engine")
     ap.add_argument("--rubasun-models", default="rubasun,llama",
                     help="with --rubasun: which of the two models to run (for profiles of one of them)")
+    ap.add_argument("--virusun", default="", metavar="SIZES",
+                    help="the same for the Virusun design (sizes of: 2048, 4096)")
+    ap.add_argument("--virusun-models", default="virusun,llama",
+                    help="with --virusun: which of the two models to run (for profiles of one of them)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
@@ -380,6 +434,8 @@ def main():
     per_req_pages = -(-(S + max(W, K) + slack) // page)
     if args.rubasun:
         return rubasun_beside_llama(args)
+    if args.virusun:
+        return virusun_beside_llama(args)
     if args.mixed:
         return mixed_workload(args, cfg, short)
     if args.like_reference:

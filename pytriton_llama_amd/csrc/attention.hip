@@ -281,23 +281,29 @@ __device__ __forceinline__ void load_chunk<bf16_t>(const bf16_t* __restrict__ p,
   }
 }
 
-template <typename T, int GT, int LPK>
+// Keys of size Dk, values of size Dv and ``maps`` score maps a head as in the general form of
+// the kernel above: the "kv head" of the grid is a key head (kv head, map); its query heads are
+// head * maps + map for the heads of the kv head, its values those of the kv head. LPK lanes cover
+// max(Dk, Dv). TO: the type of the result.
+template <typename T, typename TO, int GT, int LPK>
 __global__ void __launch_bounds__(256)
-attn_decode_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q, long q_stride,
+attn_decode_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__ q, long q_stride,
                    const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
                    const int32_t* __restrict__ block_table, int bt_stride,
                    float* __restrict__ part_acc, float* __restrict__ part_ml,
-                   int Hq, int Hkv, int D, int page_size, int window, float scale,
+                   int Hq, int Hkv, int maps, int Dk, int Dv, int page_size, int window, float scale,
                    int num_splits, int groups_per_kv) {
   constexpr int KPW = 64 / LPK;           // keys a wave reads per turn
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int seq = blockIdx.x;
-  const int kvh = blockIdx.y / groups_per_kv;
-  const int hg = blockIdx.y - kvh * groups_per_kv;
+  const int kh = blockIdx.y / groups_per_kv;          // key head: (kv head, map)
+  const int hg = blockIdx.y - kh * groups_per_kv;
+  const int vh = kh / maps, map = kh - vh * maps;
+  const int Hk = Hkv * maps;
   const int split = blockIdx.z;
-  const int G = Hq / Hkv;
-  const int head0 = kvh * G + hg * GT;      // first query head of this workgroup
+  const int G = (Hq / maps) / Hkv;
+  const int head0 = vh * G + hg * GT;       // first head (of Hq / maps) of this workgroup
   const int nheads = min(GT, G - hg * GT);
   const int row = q_start[seq];
   const int ctx = ctx_len[seq];
@@ -311,13 +317,13 @@ attn_decode_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q
 
   const int c = lane % LPK;                 // which 16 elements of the head this lane owns
   const int ks = lane / LPK;                // key slot within the wave
-  const bool active = c * DEC_CHUNK < D;
+  const bool active_k = c * DEC_CHUNK < Dk, active_v = c * DEC_CHUNK < Dv;
 
   float qf[GT][DEC_CHUNK];
 #pragma unroll
   for (int h = 0; h < GT; ++h) {
-    if (h < nheads && active) {
-      load_chunk<T>(q + (size_t)row * q_stride + (size_t)(head0 + h) * D + c * DEC_CHUNK, qf[h]);
+    if (h < nheads && active_k) {
+      load_chunk<T>(q + (size_t)row * q_stride + (size_t)((head0 + h) * maps + map) * Dk + c * DEC_CHUNK, qf[h]);
 #pragma unroll
       for (int j = 0; j < DEC_CHUNK; ++j) qf[h][j] *= scale;
     } else {
@@ -337,14 +343,15 @@ attn_decode_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q
     const int kp = kb + ks;
     const bool valid = kp < k_end;
     float kf[DEC_CHUNK], vf[DEC_CHUNK];
-    if (valid && active) {
-      const int page = bt[kp / page_size];
-      const size_t idx = (((size_t)page * Hkv + kvh) * page_size + (kp % page_size)) * D + c * DEC_CHUNK;
-      load_chunk<T>(k_cache + idx, kf);
-      load_chunk<T>(v_cache + idx, vf);
-    } else {
 #pragma unroll
-      for (int j = 0; j < DEC_CHUNK; ++j) { kf[j] = 0.f; vf[j] = 0.f; }
+    for (int j = 0; j < DEC_CHUNK; ++j) { kf[j] = 0.f; vf[j] = 0.f; }
+    if (valid) {
+      const int page = bt[kp / page_size];
+      const int in_page = kp % page_size;
+      if (active_k)
+        load_chunk<T>(k_cache + (((size_t)page * Hk + kh) * page_size + in_page) * Dk + c * DEC_CHUNK, kf);
+      if (active_v)
+        load_chunk<T>(v_cache + (((size_t)page * Hkv + vh) * page_size + in_page) * Dv + c * DEC_CHUNK, vf);
     }
 #pragma unroll
     for (int h = 0; h < GT; ++h) {
@@ -389,19 +396,21 @@ attn_decode_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q
 
   // merge the four waves through LDS
   extern __shared__ float lds[];
-  float* w_acc = lds;                         // [4][GT][D]
-  float* w_ml = lds + 4 * GT * D;             // [4][GT][2]
-  if (ks == 0 && active) {
+  float* w_acc = lds;                         // [4][GT][Dv]
+  float* w_ml = lds + 4 * GT * Dv;            // [4][GT][2]
+  if (ks == 0) {
 #pragma unroll
     for (int h = 0; h < GT; ++h) {
+      if (active_v) {
 #pragma unroll
-      for (int j = 0; j < DEC_CHUNK; ++j) w_acc[(wave * GT + h) * D + c * DEC_CHUNK + j] = acc[h][j];
+        for (int j = 0; j < DEC_CHUNK; ++j) w_acc[(wave * GT + h) * Dv + c * DEC_CHUNK + j] = acc[h][j];
+      }
       if (c == 0) { w_ml[(wave * GT + h) * 2] = m[h]; w_ml[(wave * GT + h) * 2 + 1] = l[h]; }
     }
   }
   __syncthreads();
-  for (int i = tid; i < nheads * D; i += 256) {
-    const int h = i / D, d = i - h * D;
+  for (int i = tid; i < nheads * Dv; i += 256) {
+    const int h = i / Dv, d = i - h * Dv;
     float mn = -INFINITY;
 #pragma unroll
     for (int w = 0; w < 4; ++w) mn = fmaxf(mn, w_ml[(w * GT + h) * 2]);
@@ -411,14 +420,14 @@ attn_decode_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q
     for (int w = 0; w < 4; ++w) {
       const float f = expf(w_ml[(w * GT + h) * 2] - ms);
       ll += w_ml[(w * GT + h) * 2 + 1] * f;
-      a += w_acc[(w * GT + h) * D + d] * f;
+      a += w_acc[(w * GT + h) * Dv + d] * f;
     }
-    const int head = head0 + h;
+    const int head = (head0 + h) * maps + map;
     if (num_splits == 1) {
-      out[(size_t)row * out_stride + (size_t)head * D + d] = from_float<T>(ll > 0.f ? a / ll : 0.f);
+      out[(size_t)row * out_stride + (size_t)head * Dv + d] = from_float<TO>(ll > 0.f ? a / ll : 0.f);
     } else {
       const size_t pi = ((size_t)seq * Hq + head) * num_splits + split;
-      part_acc[pi * D + d] = a;
+      part_acc[pi * Dv + d] = a;
       if (d == 0) { part_ml[pi * 2] = mn; part_ml[pi * 2 + 1] = ll; }
     }
   }
@@ -471,33 +480,74 @@ attn_decode_merge_kernel(T* __restrict__ out, long out_stride, const int32_t* __
   }
 }
 
-template <typename T, int LPK>
+template <typename T, typename TO, int LPK>
 static int launch_decode(void* out, long out_stride, const void* q, long q_stride,
                          const void* k_cache, const void* v_cache, const int32_t* q_start,
                          const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
-                         float* part_acc, float* part_ml, int n_seq, int Hq, int Hkv, int D,
-                         int page_size, int window, float scale, int num_splits, hipStream_t stream) {
+                         float* part_acc, float* part_ml, int n_seq, int Hq, int Hkv, int maps, int Dk,
+                         int Dv, int page_size, int window, float scale, int num_splits,
+                         hipStream_t stream) {
   constexpr int GT = 4;
-  const int G = Hq / Hkv;
+  const int G = (Hq / maps) / Hkv;
   const int groups = (G + GT - 1) / GT;
-  dim3 grid(n_seq, Hkv * groups, num_splits);
-  const size_t lds = (size_t)(4 * GT * D + 4 * GT * 2) * sizeof(float);
-  attn_decode_kernel<T, GT, LPK><<<grid, 256, lds, stream>>>(
-      (T*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, q_start,
-      ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv, D, page_size, window, scale,
-      num_splits, groups);
+  dim3 grid(n_seq, Hkv * maps * groups, num_splits);
+  const size_t lds = (size_t)(4 * GT * Dv + 4 * GT * 2) * sizeof(float);
+  attn_decode_kernel<T, TO, GT, LPK><<<grid, 256, lds, stream>>>(
+      (TO*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, q_start,
+      ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv, maps, Dk, Dv, page_size, window,
+      scale, num_splits, groups);
   if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
   if (num_splits > 1) {
     dim3 mgrid(n_seq, Hq);
-    attn_decode_merge_kernel<T><<<mgrid, 64, 0, stream>>>((T*)out, out_stride, q_start, part_acc,
-                                                         part_ml, Hq, D, num_splits);
+    attn_decode_merge_kernel<TO><<<mgrid, 64, 0, stream>>>((TO*)out, out_stride, q_start, part_acc,
+                                                          part_ml, Hq, Dv, num_splits);
   }
   return ptl_launch_status();
 }
 
-// Sequences 0..n_seq-1 of the tables each bring one query token (row q_start[s]).
-// part_acc [n_seq, Hq, num_splits, D] and part_ml [n_seq, Hq, num_splits, 2] are
+// Sequences 0..n_seq-1 of the tables each bring one query token (row q_start[s]). q [T, Hq, Dk]
+// with Hq = heads * maps, k_cache [pages, Hkv * maps, page_size, Dk], v_cache [pages, Hkv,
+// page_size, Dv], out [T, Hq, Dv] of the caches' type or (out_f32) float32.
+// part_acc [n_seq, Hq, num_splits, Dv] and part_ml [n_seq, Hq, num_splits, 2] are
 // float32 workspaces of the caller (unused when num_splits == 1).
+extern "C" int ptl_attention_decode_kv(void* out, long out_stride, int out_f32, const void* q,
+                                       long q_stride, const void* k_cache, const void* v_cache,
+                                       const int32_t* q_start, const int32_t* ctx_len,
+                                       const int32_t* block_table, int bt_stride, float* part_acc,
+                                       float* part_ml, int n_seq, int Hq, int Hkv, int maps, int Dk,
+                                       int Dv, int page_size, int window, float scale, int num_splits,
+                                       int dtype, hipStream_t stream) {
+  if (n_seq <= 0) return PTL_OK;
+  if (Hq <= 0 || Hkv <= 0 || maps <= 0 || Hq % maps || (Hq / maps) % Hkv || Dk <= 0 || Dk % 16 ||
+      Dk > 256 || Dv <= 0 || Dv % 16 || Dv > 256 || page_size <= 0 || num_splits < 1 ||
+      num_splits > 1024 || (num_splits > 1 && (!part_acc || !part_ml)))
+    return PTL_ERR_ARG;
+  const int chunks = (Dk > Dv ? Dk : Dv) / 16;
+  int lpk = 1;
+  while (lpk < chunks) lpk <<= 1;
+#define GO(T, TO, L) launch_decode<T, TO, L>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
+                                             ctx_len, block_table, bt_stride, part_acc, part_ml,    \
+                                             n_seq, Hq, Hkv, maps, Dk, Dv, page_size, window, scale, \
+                                             num_splits, stream)
+#define BY_LPK(T, TO)                                                                              \
+  switch (lpk) {                                                                                   \
+    case 1: return GO(T, TO, 1);                                                                   \
+    case 2: return GO(T, TO, 2);                                                                   \
+    case 4: return GO(T, TO, 4);                                                                   \
+    case 8: return GO(T, TO, 8);                                                                   \
+    default: return GO(T, TO, 16);                                                                 \
+  }
+  if (dtype == PTL_DTYPE_F32) { BY_LPK(float, float) }
+  if (dtype == PTL_DTYPE_BF16) {
+    if (out_f32) { BY_LPK(bf16_t, float) }
+    BY_LPK(bf16_t, bf16_t)
+  }
+#undef BY_LPK
+#undef GO
+  return PTL_ERR_ARG;
+}
+
+// Keys and values of one size, one score map a head.
 extern "C" int ptl_attention_decode(void* out, long out_stride, const void* q, long q_stride,
                                     const void* k_cache, const void* v_cache,
                                     const int32_t* q_start, const int32_t* ctx_len,
@@ -505,29 +555,9 @@ extern "C" int ptl_attention_decode(void* out, long out_stride, const void* q, l
                                     float* part_ml, int n_seq, int Hq, int Hkv, int D, int page_size,
                                     int window, float scale, int num_splits, int dtype,
                                     hipStream_t stream) {
-  if (n_seq <= 0) return PTL_OK;
-  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || D % 16 || D > 256 || page_size <= 0 ||
-      num_splits < 1 || num_splits > 1024 || (num_splits > 1 && (!part_acc || !part_ml)))
-    return PTL_ERR_ARG;
-  const int chunks = D / 16;
-  int lpk = 1;
-  while (lpk < chunks) lpk <<= 1;
-#define GO(T, L) launch_decode<T, L>(out, out_stride, q, q_stride, k_cache, v_cache, q_start,      \
-                                     ctx_len, block_table, bt_stride, part_acc, part_ml, n_seq,    \
-                                     Hq, Hkv, D, page_size, window, scale, num_splits, stream)
-#define BY_LPK(T)                                                                                  \
-  switch (lpk) {                                                                                   \
-    case 1: return GO(T, 1);                                                                       \
-    case 2: return GO(T, 2);                                                                       \
-    case 4: return GO(T, 4);                                                                       \
-    case 8: return GO(T, 8);                                                                       \
-    default: return GO(T, 16);                                                                     \
-  }
-  if (dtype == PTL_DTYPE_F32) { BY_LPK(float) }
-  if (dtype == PTL_DTYPE_BF16) { BY_LPK(bf16_t) }
-#undef BY_LPK
-#undef GO
-  return PTL_ERR_ARG;
+  return ptl_attention_decode_kv(out, out_stride, 0, q, q_stride, k_cache, v_cache, q_start, ctx_len,
+                                 block_table, bt_stride, part_acc, part_ml, n_seq, Hq, Hkv, 1, D, D,
+                                 page_size, window, scale, num_splits, dtype, stream);
 }
 
 // ===========================================================================

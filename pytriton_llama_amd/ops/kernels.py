@@ -1146,6 +1146,52 @@ def attention_generic_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tens
         _dtype_code(q), _stream()), "attention")
 
 
+def attention_decode_kv_fits(Dk: int, Dv: int) -> bool:
+    """Whether the split-KV kernel takes keys of size Dk with values of size Dv."""
+    return Dk % 16 == 0 and Dv % 16 == 0 and 0 < Dk <= 256 and 0 < Dv <= 256
+
+
+def attention_decode_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                        q_start: torch.Tensor, ctx_len: torch.Tensor, block_table: torch.Tensor, n_seq: int,
+                        scale: float, maps: int = 1, num_splits: int = 1, window: int = 0) -> None:
+    """Split-KV attention of the first ``n_seq`` sequences of the tables, each of which brings one
+    query token, with keys and values of different sizes and ``maps`` score maps a head (shapes as
+    for attention_generic_kv; sizes in steps of 16 up to 256)."""
+    _need_gpu(out, q, k_cache, v_cache, q_start, ctx_len, block_table)
+    if q.dim() != 3 or k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelError("attention_decode_kv: q [T, Hq, Dk], caches [pages, heads, page_size, size]")
+    T, Hq, Dk = q.shape
+    pages, Hk, page_size, _ = k_cache.shape
+    Hkv, Dv = v_cache.shape[1], v_cache.shape[3]
+    if (k_cache.shape[3] != Dk or v_cache.shape[0] != pages or v_cache.shape[2] != page_size
+            or maps <= 0 or Hk != Hkv * maps or Hq % maps or (Hq // maps) % Hkv):
+        raise KernelError("attention_decode_kv: q, keys and values do not fit each other")
+    if not attention_decode_kv_fits(Dk, Dv):
+        raise KernelError(f"attention_decode_kv: sizes {Dk}, {Dv} are not multiples of 16 up to 256")
+    if out.shape != (T, Hq, Dv) or not out.is_contiguous() or not q.is_contiguous() or q.data_ptr() % 16:
+        raise KernelError(f"attention_decode_kv: q and out [{T}, {Hq}, {Dv}] must be contiguous and aligned")
+    if not (q.dtype == k_cache.dtype == v_cache.dtype) or out.dtype not in (q.dtype, torch.float32):
+        raise KernelError("attention_decode_kv: q and the caches share one dtype; out has it, or float32")
+    if not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("attention_decode_kv: caches must be contiguous")
+    _i32(q_start, "q_start")
+    _i32(ctx_len, "ctx_len")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("attention_decode_kv: block_table must be int32 [n, max_pages]")
+    if n_seq > ctx_len.numel() or q_start.numel() < n_seq + 1 or block_table.shape[0] < n_seq or num_splits < 1:
+        raise KernelError("attention_decode_kv: tables are shorter than n_seq, or no splits")
+    part_acc = part_ml = None
+    if num_splits > 1:
+        part_acc = torch.empty((n_seq, Hq, num_splits, Dv), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_seq, Hq, num_splits, 2), dtype=torch.float32, device=q.device)
+    _check(library.load("attention").ptl_attention_decode_kv(
+        _ptr(out), ctypes.c_long(out.stride(0)), int(out.dtype == torch.float32 and q.dtype != torch.float32),
+        _ptr(q), ctypes.c_long(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len),
+        _ptr(block_table), int(block_table.stride(0)), _ptr(part_acc), _ptr(part_ml), int(n_seq), Hq, Hkv,
+        int(maps), Dk, Dv, page_size, int(window), ctypes.c_float(scale), int(num_splits), _dtype_code(q),
+        _stream()), "attention_decode_kv")
+
+
 # ---------------------------------------------------------------------------
 # Normed queries and keys, results normed head by head (csrc/prepare.hip)
 NORM_NONE, NORM_HEAD, NORM_WHOLE = 0, 1, 2

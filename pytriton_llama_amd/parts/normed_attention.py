@@ -8,7 +8,7 @@ from typing import List, Optional
 import torch
 
 from .. import ops
-from .attention import ALL_16
+from .attention import ALL_16, PORTIONS_16
 from .base import PagedSpec, PagedTensor, ParamSource, Part, PendingSum, as_tensor, place, register_part
 from .linear import LINEAR_LIBRARIES, decode_copy, linear
 from .rotary import ramp_inv_freq
@@ -96,10 +96,37 @@ class NormedAttention(Part):
         self.q_bias = self.k_bias = self.v_bias = self.o_bias = None
         self.q_weight = self.k_weight = self.inv_freq = None
         self.lam = 0.0
+        self.force_decode_splits = 0        # tests set it to try other splits
         self.kernel_libraries = ("attention", "prepare", "stream") + LINEAR_LIBRARIES
 
     def work_lists(self):
-        return (ALL_16,)
+        return (ALL_16, PORTIONS_16)
+
+    def decode_splits(self, ctx, n_dec: int, device) -> int:
+        """How many workgroups share one decoding sequence's keys: enough to fill the compute
+        units about four times over, never finer than one turn of a workgroup."""
+        if self.force_decode_splits:
+            return self.force_decode_splits
+        lpk = 1
+        while lpk * 16 < max(self.dim, self.vdim):
+            lpk <<= 1
+        turn = 2 * (256 // lpk)
+        per_kv = self.num_heads // self.num_kv_heads
+        base = max(1, n_dec * self.num_kv_heads * self.maps * (-(-per_kv // 4)))
+        want = -(-4 * ops.compute_units(device) // base)
+        return max(1, min(want, -(-max(ctx.ctx_lens[:n_dec]) // turn), 64))
+
+    def attend(self, a, q, cache, ctx, group) -> None:
+        """Leading sequences of one token: the split-KV kernel; the rest: 16-row blocks."""
+        n_dec = ctx.num_decode_seqs if ops.attention_decode_kv_fits(self.dim, self.vdim) else 0
+        if n_dec:
+            ops.attention_decode_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table, n_dec,
+                                    self.scale, self.maps, self.decode_splits(ctx, n_dec, q.device))
+        if n_dec == ctx.num_seqs:
+            return
+        ws, wo = ctx.work[PORTIONS_16 if n_dec else ALL_16]
+        ops.attention_generic_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table,
+                                 ws, wo, self.scale, self.maps)
 
     def cache_spec(self):
         if not self.own_kv:
@@ -184,9 +211,7 @@ class NormedAttention(Part):
                         H * M, G * M, G, Dk, Dv, cache.page_size)
         plain = M == 1
         a = torch.empty((T, H * M, Dv), dtype=x.dtype if plain else torch.float32, device=x.device)
-        ws, wo = ctx.work[ALL_16]
-        ops.attention_generic_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table,
-                                 ws, wo, self.scale, M)
+        self.attend(a, q, cache, ctx, group)
         if plain:
             return a.view(T, H * Dv)
         out = torch.empty((T, H * Dv), dtype=x.dtype, device=x.device)

@@ -321,3 +321,48 @@ def test_norm_of_a_weighted_sum_into_the_stream(gpu_device, dtype):
         assert float((copy.double().cpu() - want).abs().max()) < (1e-5 if dtype == torch.float32 else 3e-2)
     out = ops.stream_rmsnorm(dev(stream), dev(w), eps, dtype)
     assert float((out.double().cpu() - pv.rms(stream, eps) * w).abs().max()) < (1e-5 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("maps,H,G,Dk,Dv", [(1, 6, 3, 32, 48), (2, 4, 2, 48, 96), (2, 10, 2, 16, 16), (1, 2, 1, 144, 32)])
+@pytest.mark.parametrize("splits", [1, 3, 8])
+def test_decoding_attention_with_keys_split_over_workgroups(gpu_device, dtype, maps, H, G, Dk, Dv, splits):
+    """Single query tokens of three sequences (1, 130 and 333 keys; pages in shuffled order), the
+    keys of each cut into ``splits`` parts; for one head the key at a page's last place is made to
+    stand out."""
+    from pytriton_llama_amd import ops
+    torch.manual_seed(19)
+    P, pages, scale = 8, 80, 0.25
+    lens = [1, 130, 333]
+    order = torch.randperm(pages).tolist()
+    k_pool = torch.randn(pages, G * maps, P, Dk, dtype=torch.float64) * 5
+    v_pool = torch.randn(pages, G, P, Dv, dtype=torch.float64) * 5
+    bt = torch.full((3, -(-max(lens) // P)), -1, dtype=torch.int32)
+    qs, want, at = [], [], 0
+    for r, n in enumerate(lens):
+        k = torch.randn(n, G * maps, Dk, dtype=torch.float64)
+        v = torch.randn(n, G, Dv, dtype=torch.float64)
+        q = torch.randn(1, H * maps, Dk, dtype=torch.float64)
+        if n > P:
+            k[P * 2 - 1] *= 3.0
+            q[0, 0] = k[P * 2 - 1, 0] * 2.0
+        if dtype == torch.bfloat16:
+            q, k, v = (t.bfloat16().double() for t in (q, k, v))
+        out = torch.zeros(1, H * maps, Dv, dtype=torch.float64)
+        for j in range(H * maps):
+            vh = (j // maps) // (H // G)
+            out[0, j] = torch.softmax((q[0, j] @ k[:, vh * maps + j % maps].T) * scale, -1) @ v[:, vh]
+        table = order[at:at + -(-n // P)]
+        at += len(table)
+        bt[r, :len(table)] = torch.tensor(table, dtype=torch.int32)
+        for i in range(n):
+            k_pool[table[i // P], :, i % P] = k[i]
+            v_pool[table[i // P], :, i % P] = v[i]
+        qs.append(q), want.append(out)
+    want = torch.cat(want)
+    for out_dtype in ([torch.float32] if dtype == torch.float32 else [torch.float32, torch.bfloat16]):
+        out = torch.empty(3, H * maps, Dv, dtype=out_dtype, device="cuda")
+        ops.attention_decode_kv(out, dev(torch.cat(qs), dtype), dev(k_pool, dtype), dev(v_pool, dtype),
+                                i32([0, 1, 2, 3]), i32(lens), bt.cuda(), 3, scale, maps, splits)
+        tol = 2e-5 if out_dtype == torch.float32 else 1e-2
+        assert float((out.double().cpu() - want).abs().max()) < tol * float(want.abs().max())
