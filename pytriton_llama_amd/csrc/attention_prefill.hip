@@ -33,6 +33,12 @@
 // stabiliser, not a result: it follows the scores only when they pass it by more
 // than 8 (in the exponent's units), so that what is kept is rescaled rarely.
 // Needs D % 32 == 0, D <= 128, a page size that is a power of two.
+//
+// Keys of size DK and values of size DV need not be alike (both multiples of 32 up to 128), and
+// a head may come in several score maps over one set of values, as in the general form of the
+// vector kernel (attention.hip): query head j is map j % maps of head j / maps and reads key
+// head (kv head) * maps + j % maps and the values of its kv head. The result is bfloat16, or
+// float32 for one that is combined further before it is rounded.
 // ===========================================================================
 
 #define PF_BN 64
@@ -47,30 +53,43 @@ __device__ __forceinline__ s16x4_t lds_read_tr16(const bf16_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)p);
 }
 
-// RT: 16-row query tiles per wave; the workgroup takes 64 * RT query rows.
-template <int NDT, int RT>
-__global__ void __launch_bounds__(256, NDT <= 2 ? 3 : 2)
-attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
+template <typename TO> __device__ __forceinline__ void store4(TO* p, const float* v);
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float* v) {
+  union { uint2 u; bf16_t e[4]; } rr;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) rr.e[i] = float_to_bf16(v[i]);
+  *reinterpret_cast<uint2*>(p) = rr.u;
+}
+template <> __device__ __forceinline__ void store4<float>(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// NDK, NDV: key and value sizes in units of 32. RT: 16-row query tiles per wave; the workgroup
+// takes 64 * RT query rows.
+template <int NDK, int NDV, int RT, typename TO>
+__global__ void __launch_bounds__(256, (NDK + NDV) <= 4 ? 3 : 2)
+attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
                          long q_stride, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ q_start,
                          const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ block_table,
                          int bt_stride, const int32_t* __restrict__ work_seq,
-                         const int32_t* __restrict__ work_qoff, int n_work, int Hq, int Hkv,
+                         const int32_t* __restrict__ work_qoff, int n_work, int Hq, int Hkv, int maps,
                          int page_size, int page_shift, int window, float scale_log2) {
-  constexpr int D = 32 * NDT;
+  constexpr int DK = 32 * NDK, DV = 32 * NDV;
   constexpr int PBM = 64 * RT;
-  constexpr int CPR = D / 8;           // 16-byte chunks per row
-  constexpr int NCH = PF_BN * CPR / 256;   // chunks of a tile per thread
+  constexpr int CPRK = DK / 8, CPRV = DV / 8;      // 16-byte chunks per row
+  constexpr int NCHK = PF_BN * CPRK / 256, NCHV = PF_BN * CPRV / 256;   // chunks of a tile per thread
   // Tiles lie in LDS as rows of D elements without padding; the 16-byte chunks of a row are
   // permuted (chunk c of row r lies at c ^ swz(r)) so that neither the row-wise reads of the
   // first product nor the transposing reads of the second meet in a bank. Two buffers each,
   // as separate arrays: the compiler then knows that a load into one does not touch the other.
-  constexpr bool SW8 = CPR % 8 == 0;
-  __shared__ __attribute__((aligned(1024))) bf16_t Ks0[PF_BN * D];
-  __shared__ __attribute__((aligned(1024))) bf16_t Ks1[PF_BN * D];
-  __shared__ __attribute__((aligned(1024))) bf16_t Vs0[PF_BN * D];
-  __shared__ __attribute__((aligned(1024))) bf16_t Vs1[PF_BN * D];
-  auto swz = [](int row) { return SW8 ? (row & 7) : ((row >> 1) & 3); };
+  constexpr bool SW8K = CPRK % 8 == 0, SW8V = CPRV % 8 == 0;
+  __shared__ __attribute__((aligned(1024))) bf16_t Ks0[PF_BN * DK];
+  __shared__ __attribute__((aligned(1024))) bf16_t Ks1[PF_BN * DK];
+  __shared__ __attribute__((aligned(1024))) bf16_t Vs0[PF_BN * DV];
+  __shared__ __attribute__((aligned(1024))) bf16_t Vs1[PF_BN * DV];
+  auto swzk = [](int row) { return SW8K ? (row & 7) : ((row >> 1) & 3); };
+  auto swzv = [](int row) { return SW8V ? (row & 7) : ((row >> 1) & 3); };
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 15, lg = lane >> 4;
@@ -94,39 +113,40 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
   const int cached = ctx - qlen;
   const int rows = min(PBM, qlen - qoff);
   if (rows <= 0) continue;
-  const int kvh = head / (Hq / Hkv);
+  const int vh = (head / maps) / ((Hq / maps) / Hkv);      // value head
+  const int kh = vh * maps + head % maps;                   // key head (of Hkv * maps)
   const int32_t* bt = block_table + (size_t)seq * bt_stride;
   const int first_q = cached + qoff;
 
   // query rows of this lane: tile r covers rows 16*(RT*wave + r) .. +15 of the block
   int qpos[RT];
   bool row_ok[RT];
-  Frag8 qf[RT][NDT];
+  Frag8 qf[RT][NDK];
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
     const int my_row = 16 * (RT * wave + r) + ln;
     row_ok[r] = my_row < rows;
     const int qrow = row_ok[r] ? my_row : 0;       // rows past the end repeat row 0; never stored
     qpos[r] = first_q + qrow;
-    const bf16_t* qp = q + (size_t)(qs + qoff + qrow) * q_stride + (size_t)head * D + 8 * lg;
+    const bf16_t* qp = q + (size_t)(qs + qoff + qrow) * q_stride + (size_t)head * DK + 8 * lg;
 #pragma unroll
-    for (int kk = 0; kk < NDT; ++kk) qf[r][kk].u = *reinterpret_cast<const uint4*>(qp + 32 * kk);
+    for (int kk = 0; kk < NDK; ++kk) qf[r][kk].u = *reinterpret_cast<const uint4*>(qp + 32 * kk);
   }
   const int wave_first_row = 16 * RT * wave;
   const bool wave_has_rows = wave_first_row < rows;
   const int wave_min_q = first_q + (wave_has_rows ? wave_first_row : 0);
   const int wave_max_q = first_q + min(rows, wave_first_row + 16 * RT) - 1;
 
-  // The softmax denominator: o[r][2 NDT] is one more tile of the second product, whose
+  // The softmax denominator: o[r][2 NDV] is one more tile of the second product, whose
   // "values" are all one; it sums the probabilities as the product sees them (rounded to
   // bfloat16; float32 sums) and is rescaled with the numerators.
-  f32x4_t o[RT][2 * NDT + 1];
+  f32x4_t o[RT][2 * NDV + 1];
   float m_run[RT];
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
     m_run[r] = -INFINITY;
 #pragma unroll
-    for (int t = 0; t <= 2 * NDT; ++t) o[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t <= 2 * NDV; ++t) o[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
   Frag8 ones;
 #pragma unroll
@@ -144,18 +164,25 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
   // This thread's chunks of a tile. A wave's load instruction fills 64 consecutive 16-byte
   // slots of LDS, lane l the l-th; slot s holds row s / CPR, chunk (s % CPR) ^ swz(row).
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  int crow[NCH], ccol[NCH];
+  int crowk[NCHK], ccolk[NCHK], crowv[NCHV], ccolv[NCHV];
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int slot = 64 * (wave_u * NCH + i) + lane;
-    crow[i] = slot / CPR;
-    ccol[i] = ((slot - crow[i] * CPR) ^ swz(crow[i])) * 8;
+  for (int i = 0; i < NCHK; ++i) {
+    const int slot = 64 * (wave_u * NCHK + i) + lane;
+    crowk[i] = slot / CPRK;
+    ccolk[i] = ((slot - crowk[i] * CPRK) ^ swzk(crowk[i])) * 8;
   }
-  const bf16_t* k_head = k_cache + (size_t)kvh * page_size * D;
-  const bf16_t* v_head = v_cache + (size_t)kvh * page_size * D;
+#pragma unroll
+  for (int i = 0; i < NCHV; ++i) {
+    const int slot = 64 * (wave_u * NCHV + i) + lane;
+    crowv[i] = slot / CPRV;
+    ccolv[i] = ((slot - crowv[i] * CPRV) ^ swzv(crowv[i])) * 8;
+  }
+  const bf16_t* k_head = k_cache + (size_t)kh * page_size * DK;
+  const bf16_t* v_head = v_cache + (size_t)vh * page_size * DV;
 
-  int pg[NCH];                  // pages of the chunks' rows, read one tile ahead of the rows
-  const uint32_t page_bytes = (uint32_t)Hkv * page_size * D * 2;     // < 4 GiB, checked by the host
+  int pgk[NCHK], pgv[NCHV];     // pages of the chunks' rows, read one tile ahead of the rows
+  const uint32_t page_bytes_k = (uint32_t)Hkv * maps * page_size * DK * 2;     // < 4 GiB, checked by the host
+  const uint32_t page_bytes_v = (uint32_t)Hkv * page_size * DV * 2;
   const int page_mask = page_size - 1;                                // page sizes are powers of two
   // a tile that lies wholly inside the keys this block sees needs no tests (uniform)
   auto whole = [&](int t) {
@@ -166,61 +193,65 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
     const int k0 = k_begin + t * PF_BN;
     if (whole(t)) {
 #pragma unroll
-      for (int i = 0; i < NCH; ++i) pg[i] = bt[(k0 + crow[i]) >> page_shift];
+      for (int i = 0; i < NCHK; ++i) pgk[i] = bt[(k0 + crowk[i]) >> page_shift];
+#pragma unroll
+      for (int i = 0; i < NCHV; ++i) pgv[i] = bt[(k0 + crowv[i]) >> page_shift];
     } else {
 #pragma unroll
-      for (int i = 0; i < NCH; ++i) {
-        const int kp = k0 + crow[i];
-        pg[i] = -1;
-        if (t < n_tiles && kp >= k_lo && kp < k_end) pg[i] = bt[kp >> page_shift];
+      for (int i = 0; i < NCHK; ++i) {
+        const int kp = k0 + crowk[i];
+        pgk[i] = -1;
+        if (t < n_tiles && kp >= k_lo && kp < k_end) pgk[i] = bt[kp >> page_shift];
+      }
+#pragma unroll
+      for (int i = 0; i < NCHV; ++i) {
+        const int kp = k0 + crowv[i];
+        pgv[i] = -1;
+        if (t < n_tiles && kp >= k_lo && kp < k_end) pgv[i] = bt[kp >> page_shift];
       }
     }
   };
   // global memory -> LDS without a register in between (global_load_lds_dwordx4): every lane
   // names its own 16 bytes of global memory, the wave's 64 chunks land side by side in LDS
-  auto to_lds = [&](const bf16_t* base, uint64_t at, bf16_t* tile_lds, int i) {
+  auto to_lds = [&](const bf16_t* base, uint64_t at, bf16_t* tile_lds, int chunk) {
     __builtin_amdgcn_global_load_lds(
         (const __attribute__((address_space(1))) void*)(reinterpret_cast<const char*>(base) + at),
-        (__attribute__((address_space(3))) void*)(tile_lds + 512 * (wave_u * NCH + i)), 16, 0, 0);
+        (__attribute__((address_space(3))) void*)(tile_lds + 512 * chunk), 16, 0, 0);
   };
   auto fetch = [&](int t, bf16_t* Kb, bf16_t* Vb) {
     const int k0 = k_begin + t * PF_BN;
-    if (whole(t)) {
+    const bool all = whole(t);
 #pragma unroll
-      for (int i = 0; i < NCH; ++i) {
-        const uint32_t in_page = (uint32_t)(((k0 + crow[i]) & page_mask) * D + ccol[i]) * 2;
-        const uint64_t at = (uint64_t)(uint32_t)pg[i] * page_bytes + in_page;
-        to_lds(k_head, at, Kb, i);
-        to_lds(v_head, at, Vb, i);
+    for (int i = 0; i < NCHK; ++i) {
+      if (all || pgk[i] >= 0) {
+        const uint32_t in_page = (uint32_t)(((k0 + crowk[i]) & page_mask) * DK + ccolk[i]) * 2;
+        to_lds(k_head, (uint64_t)(uint32_t)pgk[i] * page_bytes_k + in_page, Kb, wave_u * NCHK + i);
+      } else {                                    // rows outside the keys read as zeros
+        *reinterpret_cast<uint4*>(Kb + 8 * (64 * (wave_u * NCHK + i) + lane)) = make_uint4(0, 0, 0, 0);
       }
-    } else {
+    }
 #pragma unroll
-      for (int i = 0; i < NCH; ++i) {
-        if (pg[i] >= 0) {
-          const uint32_t in_page = (uint32_t)(((k0 + crow[i]) & page_mask) * D + ccol[i]) * 2;
-          const uint64_t at = (uint64_t)(uint32_t)pg[i] * page_bytes + in_page;
-          to_lds(k_head, at, Kb, i);
-          to_lds(v_head, at, Vb, i);
-        } else {                                  // rows outside the keys read as zeros
-          const int slot = 64 * (wave_u * NCH + i) + lane;
-          *reinterpret_cast<uint4*>(Kb + 8 * slot) = make_uint4(0, 0, 0, 0);
-          *reinterpret_cast<uint4*>(Vb + 8 * slot) = make_uint4(0, 0, 0, 0);
-        }
+    for (int i = 0; i < NCHV; ++i) {
+      if (all || pgv[i] >= 0) {
+        const uint32_t in_page = (uint32_t)(((k0 + crowv[i]) & page_mask) * DV + ccolv[i]) * 2;
+        to_lds(v_head, (uint64_t)(uint32_t)pgv[i] * page_bytes_v + in_page, Vb, wave_u * NCHV + i);
+      } else {
+        *reinterpret_cast<uint4*>(Vb + 8 * (64 * (wave_u * NCHV + i) + lane)) = make_uint4(0, 0, 0, 0);
       }
     }
   };
   // where this lane reads: the first product takes row 16 kt + ln, chunk 4 kk + lg; the second
   // points at row 32 half + 16 j + 4 lg + ln / 4, elements 16 dt + 4 (ln % 4) .. +3
-  int k_at[NDT], v_at[2 * NDT];
+  int k_at[NDK], v_at[2 * NDV];
   {
-    const int sw = swz(ln);
+    const int sw = swzk(ln);
 #pragma unroll
-    for (int kk = 0; kk < NDT; ++kk) k_at[kk] = ln * D + 8 * ((4 * kk + lg) ^ sw);
+    for (int kk = 0; kk < NDK; ++kk) k_at[kk] = ln * DK + 8 * ((4 * kk + lg) ^ sw);
     const int vrow = 4 * lg + (ln >> 2);
-    const int vsw = swz(vrow);
+    const int vsw = swzv(vrow);
 #pragma unroll
-    for (int dt = 0; dt < 2 * NDT; ++dt)
-      v_at[dt] = vrow * D + 8 * ((2 * dt + ((ln & 3) >> 1)) ^ vsw) + 4 * (ln & 1);
+    for (int dt = 0; dt < 2 * NDV; ++dt)
+      v_at[dt] = vrow * DV + 8 * ((2 * dt + ((ln & 3) >> 1)) ^ vsw) + 4 * (ln & 1);
   }
 
   // one key tile for this wave's rows; MASKED: the tile touches the diagonal, the end of the
@@ -233,9 +264,9 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
 #pragma unroll
       for (int r = 0; r < RT; ++r) st[r][kt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < NDT; ++kk) {
+      for (int kk = 0; kk < NDK; ++kk) {
         Frag8 a;
-        a.u = *reinterpret_cast<const uint4*>(Kb + 16 * kt * D + k_at[kk]);
+        a.u = *reinterpret_cast<const uint4*>(Kb + 16 * kt * DK + k_at[kk]);
 #pragma unroll
         for (int r = 0; r < RT; ++r)
           st[r][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[r][kk].v, st[r][kt], 0, 0, 0);
@@ -270,7 +301,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
         const float alpha = __builtin_amdgcn_exp2f((m_run[r] - tmax) * scale_log2);
         m_run[r] = tmax;
 #pragma unroll
-        for (int t = 0; t <= 2 * NDT; ++t) {
+        for (int t = 0; t <= 2 * NDV; ++t) {
           o[r][t][0] *= alpha; o[r][t][1] *= alpha; o[r][t][2] *= alpha; o[r][t][3] *= alpha;
         }
       }
@@ -291,10 +322,10 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
 #pragma unroll
     for (int half = 0; half < 2; ++half)
 #pragma unroll
-      for (int dt = 0; dt < 2 * NDT; ++dt) {
+      for (int dt = 0; dt < 2 * NDV; ++dt) {
         Frag8 a;
-        a.s[0] = lds_read_tr16(Vb + (32 * half) * D + v_at[dt]);
-        a.s[1] = lds_read_tr16(Vb + (32 * half + 16) * D + v_at[dt]);
+        a.s[0] = lds_read_tr16(Vb + (32 * half) * DV + v_at[dt]);
+        a.s[1] = lds_read_tr16(Vb + (32 * half + 16) * DV + v_at[dt]);
 #pragma unroll
         for (int r = 0; r < RT; ++r)
           o[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb[r][half].v, o[r][dt], 0, 0, 0);
@@ -303,7 +334,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
     for (int half = 0; half < 2; ++half)
 #pragma unroll
       for (int r = 0; r < RT; ++r)
-        o[r][2 * NDT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[r][half].v, o[r][2 * NDT], 0, 0, 0);
+        o[r][2 * NDV] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[r][half].v, o[r][2 * NDV], 0, 0, 0);
   };
 
   // one turn: tile t + 1 sets out for the other buffer (everyone left it before the last
@@ -337,39 +368,59 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
 
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
-    const float l = o[r][2 * NDT][0];          // every row of that tile holds the column's sum
+    const float l = o[r][2 * NDV][0];          // every row of that tile holds the column's sum
     if (row_ok[r]) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;
       const int my_row = 16 * (RT * wave + r) + ln;
-      bf16_t* op = out + (size_t)(qs + qoff + my_row) * out_stride + (size_t)head * D + 4 * lg;
+      TO* op = out + (size_t)(qs + qoff + my_row) * out_stride + (size_t)head * DV + 4 * lg;
 #pragma unroll
-      for (int dt = 0; dt < 2 * NDT; ++dt) {
-        union { uint2 u; bf16_t e[4]; } rr;
+      for (int dt = 0; dt < 2 * NDV; ++dt) {
+        float rr[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) rr.e[i] = float_to_bf16(o[r][dt][i] * inv);
-        *reinterpret_cast<uint2*>(op + 16 * dt) = rr.u;
+        for (int i = 0; i < 4; ++i) rr[i] = o[r][dt][i] * inv;
+        store4<TO>(op + 16 * dt, rr);
       }
     }
   }
   }   // work items
 }
 
-template <int NDT, int RT>
+template <int NDK, int NDV, int RT, typename TO>
 static int launch_prefill_mfma(void* out, long out_stride, const void* q, long q_stride,
                                const void* k_cache, const void* v_cache, const int32_t* q_start,
                                const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
                                const int32_t* work_seq, const int32_t* work_qoff, int n_work,
-                               int n_groups, int Hq, int Hkv, int page_size, int window, float scale,
-                               hipStream_t stream) {
+                               int n_groups, int Hq, int Hkv, int maps, int page_size, int window,
+                               float scale, hipStream_t stream) {
   dim3 grid(Hq, n_groups < 65535 ? n_groups : 65535);
   int page_shift = -1;
   for (int sh = 0; sh < 31; ++sh)
     if ((1 << sh) == page_size) page_shift = sh;
-  attn_prefill_mfma_kernel<NDT, RT><<<grid, 256, 0, stream>>>(
-      (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+  attn_prefill_mfma_kernel<NDK, NDV, RT, TO><<<grid, 256, 0, stream>>>(
+      (TO*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
       (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff,
-      n_work, Hq, Hkv, page_size, page_shift, window, scale * 1.4426950408889634f);
+      n_work, Hq, Hkv, maps, page_size, page_shift, window, scale * 1.4426950408889634f);
   return ptl_launch_status();
+}
+
+// Keys and values of one size, one score map a head, bfloat16 result: the sizes every model
+// with ordinary heads brings.
+template <int RT>
+static int prefill_same_size(int nd, void* out, long out_stride, const void* q, long q_stride,
+                             const void* k_cache, const void* v_cache, const int32_t* q_start,
+                             const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
+                             const int32_t* work_seq, const int32_t* work_qoff, int n_work, int n_groups,
+                             int Hq, int Hkv, int page_size, int window, float scale, hipStream_t stream) {
+#define GO(N) launch_prefill_mfma<N, N, RT, bf16_t>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
+                                                    ctx_len, block_table, bt_stride, work_seq, work_qoff,  \
+                                                    n_work, n_groups, Hq, Hkv, 1, page_size, window, scale, stream)
+  switch (nd) {
+    case 1: return GO(1);
+    case 2: return GO(2);
+    case 3: return GO(3);
+    default: return GO(4);
+  }
+#undef GO
 }
 
 // work_seq / work_qoff list query blocks of ``block_rows`` rows (64 or 128), the longest first;
@@ -391,22 +442,53 @@ extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void
       Hq > 65535 || n_groups < 1 || n_groups > n_work || q_stride % 8 || out_stride % 4 ||
       (block_rows != 64 && block_rows != 128))
     return PTL_ERR_ARG;
-#define GO(N, R) launch_prefill_mfma<N, R>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
-                                           ctx_len, block_table, bt_stride, work_seq, work_qoff,  \
-                                           n_work, n_groups, Hq, Hkv, page_size, window, scale, stream)
-  if (block_rows == 64) {
-    switch (D / 32) {
-      case 1: return GO(1, 1);
-      case 2: return GO(2, 1);
-      case 3: return GO(3, 1);
-      default: return GO(4, 1);
-    }
+  if (block_rows == 64)
+    return prefill_same_size<1>(D / 32, out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len,
+                                block_table, bt_stride, work_seq, work_qoff, n_work, n_groups, Hq, Hkv,
+                                page_size, window, scale, stream);
+  return prefill_same_size<2>(D / 32, out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len,
+                              block_table, bt_stride, work_seq, work_qoff, n_work, n_groups, Hq, Hkv,
+                              page_size, window, scale, stream);
+}
+
+// The general form: q [T, Hq, Dk] with Hq = heads * maps, k_cache [pages, Hkv * maps, page_size,
+// Dk], v_cache [pages, Hkv, page_size, Dv], out [T, Hq, Dv] bfloat16 or (out_f32) float32; Dk and
+// Dv multiples of 32 up to 128. 64-row blocks.
+extern "C" int ptl_attention_prefill_mfma_kv(void* out, long out_stride, int out_f32, const void* q,
+                                             long q_stride, const void* k_cache, const void* v_cache,
+                                             const int32_t* q_start, const int32_t* ctx_len,
+                                             const int32_t* block_table, int bt_stride,
+                                             const int32_t* work_seq, const int32_t* work_qoff,
+                                             int n_work, int n_groups, int Hq, int Hkv, int maps, int Dk,
+                                             int Dv, int page_size, int window, float scale,
+                                             hipStream_t stream) {
+  if (n_work <= 0) return PTL_OK;
+  if (Hq <= 0 || Hkv <= 0 || maps <= 0 || Hq % maps || (Hq / maps) % Hkv || Dk % 32 || Dk <= 0 ||
+      Dk > 128 || Dv % 32 || Dv <= 0 || Dv > 128 || page_size <= 0 || (page_size & (page_size - 1)) ||
+      (long)Hkv * maps * page_size * Dk * 2 >= (1L << 32) || (long)Hkv * page_size * Dv * 2 >= (1L << 32) ||
+      Hq > 65535 || n_groups < 1 || n_groups > n_work || q_stride % 8 || out_stride % 4)
+    return PTL_ERR_ARG;
+#define GO(NK, NV, TO)                                                                                  \
+  launch_prefill_mfma<NK, NV, 1, TO>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len, \
+                                     block_table, bt_stride, work_seq, work_qoff, n_work, n_groups, Hq, \
+                                     Hkv, maps, page_size, window, scale, stream)
+#define BY_V(NK, TO)                   \
+  switch (Dv / 32) {                   \
+    case 1: return GO(NK, 1, TO);      \
+    case 2: return GO(NK, 2, TO);      \
+    case 3: return GO(NK, 3, TO);      \
+    default: return GO(NK, 4, TO);     \
   }
-  switch (D / 32) {
-    case 1: return GO(1, 2);
-    case 2: return GO(2, 2);
-    case 3: return GO(3, 2);
-    default: return GO(4, 2);
+#define BY_K(TO)                       \
+  switch (Dk / 32) {                   \
+    case 1: BY_V(1, TO)                \
+    case 2: BY_V(2, TO)                \
+    case 3: BY_V(3, TO)                \
+    default: BY_V(4, TO)               \
   }
+  if (out_f32) { BY_K(float) }
+  BY_K(bf16_t)
+#undef BY_K
+#undef BY_V
 #undef GO
 }

@@ -11,6 +11,7 @@ from .kernels import (PROBE_MFMA_FLOPS_PER_ITER, ROWS_MIN, KernelError, RowScale
                       gemm_heads_nt, latent_prepare, moe_experts, moe_route, stream_add_dyt,
                       stream_add_rmsnorm,
                       NORM_NONE, NORM_HEAD, NORM_WHOLE, GATE_NONE, GATE_SIGMOID, GATE_SILU,
-                      attention_generic_kv, attention_decode_kv, attention_decode_kv_fits, qkv_prepare, head_norm_gate, stream_add_rmsnorm_sum,
+                      attention_generic_kv, attention_decode_kv, attention_decode_kv_fits, attention_prefill_mfma_kv,
+                      attention_prefill_mfma_kv_fits, qkv_prepare, head_norm_gate, stream_add_rmsnorm_sum,
                       stream_rmsnorm, recurrent_block_floats, recurrent_state_floats, conv_prepare,
                       conv_tail_update, delta_scan, memory_scan)

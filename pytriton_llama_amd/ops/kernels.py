@@ -1146,6 +1146,59 @@ def attention_generic_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tens
         _dtype_code(q), _stream()), "attention")
 
 
+def attention_prefill_mfma_kv_fits(dtype: torch.dtype, num_kv_heads: int, maps: int, Dk: int, Dv: int,
+                                   page_size: int) -> bool:
+    """Whether the matrix-core kernel for prompt portions takes keys of size Dk with values of
+    size Dv: bfloat16, both multiples of 32 up to 128, a page size that is a power of two, pages
+    (of all heads) below 4 GiB."""
+    return (dtype == torch.bfloat16 and Dk % 32 == 0 and Dv % 32 == 0 and 0 < Dk <= 128 and 0 < Dv <= 128
+            and page_size > 0 and page_size & (page_size - 1) == 0
+            and num_kv_heads * maps * page_size * Dk * 2 < 2 ** 32 and num_kv_heads * page_size * Dv * 2 < 2 ** 32)
+
+
+def attention_prefill_mfma_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                              q_start: torch.Tensor, ctx_len: torch.Tensor, block_table: torch.Tensor,
+                              work_seq: torch.Tensor, work_qoff: torch.Tensor, scale: float, maps: int = 1,
+                              groups: int = 1, window: int = 0) -> None:
+    """The matrix-core kernel for prompt portions in its general form (csrc/attention_prefill.hip):
+    shapes as for attention_generic_kv, bfloat16 q and caches, out bfloat16 or float32; the work
+    list names 64-row blocks, ``groups`` workgroups a head share it."""
+    _need_gpu(out, q, k_cache, v_cache, q_start, ctx_len, block_table, work_seq, work_qoff)
+    if q.dim() != 3 or k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelError("attention_prefill_mfma_kv: q [T, Hq, Dk], caches [pages, heads, page_size, size]")
+    T, Hq, Dk = q.shape
+    pages, Hk, page_size, _ = k_cache.shape
+    Hkv, Dv = v_cache.shape[1], v_cache.shape[3]
+    if (k_cache.shape[3] != Dk or v_cache.shape[0] != pages or v_cache.shape[2] != page_size
+            or maps <= 0 or Hk != Hkv * maps or Hq % maps or (Hq // maps) % Hkv):
+        raise KernelError("attention_prefill_mfma_kv: q, keys and values do not fit each other")
+    if not attention_prefill_mfma_kv_fits(q.dtype, Hkv, maps, Dk, Dv, page_size):
+        raise KernelError("attention_prefill_mfma_kv: bfloat16, sizes that are multiples of 32 up to 128, a "
+                          "page size that is a power of two")
+    if (out.shape != (T, Hq, Dv) or not out.is_contiguous() or not q.is_contiguous() or q.data_ptr() % 16
+            or out.data_ptr() % 16 or out.dtype not in (torch.bfloat16, torch.float32)):
+        raise KernelError(f"attention_prefill_mfma_kv: q and out [{T}, {Hq}, {Dv}] must be contiguous and aligned")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("attention_prefill_mfma_kv: contiguous bfloat16 caches")
+    for name, t in (("q_start", q_start), ("ctx_len", ctx_len), ("work_seq", work_seq), ("work_qoff", work_qoff)):
+        _i32(t, name)
+    n = ctx_len.numel()
+    if q_start.numel() != n + 1 or work_seq.numel() != work_qoff.numel():
+        raise KernelError("attention_prefill_mfma_kv: inconsistent sequence tables")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.shape[0] < n \
+            or block_table.stride(1) != 1:
+        raise KernelError("attention_prefill_mfma_kv: block_table must be int32 [n, max_pages]")
+    n_work = int(work_seq.numel())
+    if n_work == 0:
+        return
+    _check(library.load("attention_prefill").ptl_attention_prefill_mfma_kv(
+        _ptr(out), ctypes.c_long(out.stride(0)), int(out.dtype == torch.float32), _ptr(q),
+        ctypes.c_long(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len),
+        _ptr(block_table), int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), n_work,
+        max(1, min(int(groups), n_work)), Hq, Hkv, int(maps), Dk, Dv, page_size, int(window),
+        ctypes.c_float(scale), _stream()), "attention_prefill_mfma_kv")
+
+
 def attention_decode_kv_fits(Dk: int, Dv: int) -> bool:
     """Whether the split-KV kernel takes keys of size Dk with values of size Dv."""
     return Dk % 16 == 0 and Dv % 16 == 0 and 0 < Dk <= 256 and 0 < Dv <= 256

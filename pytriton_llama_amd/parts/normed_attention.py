@@ -8,7 +8,7 @@ from typing import List, Optional
 import torch
 
 from .. import ops
-from .attention import ALL_16, PORTIONS_16
+from .attention import ALL_16, PORTIONS_16, PORTIONS_64
 from .base import PagedSpec, PagedTensor, ParamSource, Part, PendingSum, as_tensor, place, register_part
 from .linear import LINEAR_LIBRARIES, decode_copy, linear
 from .rotary import ramp_inv_freq
@@ -97,10 +97,13 @@ class NormedAttention(Part):
         self.q_weight = self.k_weight = self.inv_freq = None
         self.lam = 0.0
         self.force_decode_splits = 0        # tests set it to try other splits
-        self.kernel_libraries = ("attention", "prepare", "stream") + LINEAR_LIBRARIES
+        libs = ("attention", "prepare", "stream") + LINEAR_LIBRARIES
+        if self.dim % 32 == 0 and self.vdim % 32 == 0 and max(self.dim, self.vdim) <= 128:
+            libs += ("attention_prefill",)          # the matrix-core kernel for prompt portions
+        self.kernel_libraries = libs
 
     def work_lists(self):
-        return (ALL_16, PORTIONS_16)
+        return (ALL_16, PORTIONS_16, PORTIONS_64)
 
     def decode_splits(self, ctx, n_dec: int, device) -> int:
         """How many workgroups share one decoding sequence's keys: enough to fill the compute
@@ -117,12 +120,24 @@ class NormedAttention(Part):
         return max(1, min(want, -(-max(ctx.ctx_lens[:n_dec]) // turn), 64))
 
     def attend(self, a, q, cache, ctx, group) -> None:
-        """Leading sequences of one token: the split-KV kernel; the rest: 16-row blocks."""
+        """Leading sequences of one token: the split-KV kernel; the rest: the matrix-core kernel in
+        64-row blocks (bfloat16, sizes that are multiples of 32 up to 128) or the vector kernel in
+        16-row blocks."""
         n_dec = ctx.num_decode_seqs if ops.attention_decode_kv_fits(self.dim, self.vdim) else 0
         if n_dec:
             ops.attention_decode_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table, n_dec,
                                     self.scale, self.maps, self.decode_splits(ctx, n_dec, q.device))
         if n_dec == ctx.num_seqs:
+            return
+        if n_dec == ctx.num_decode_seqs and ops.attention_prefill_mfma_kv_fits(
+                q.dtype, self.num_kv_heads, self.maps, self.dim, self.vdim, cache.page_size):
+            ws, wo = ctx.work[PORTIONS_64]
+            # as many workgroups a head as the chip holds at once share the list of blocks
+            held = ops.compute_units(q.device) * (3 if self.dim + self.vdim <= 128 else 2)
+            t = max(1, held // (self.num_heads * self.maps))
+            blocks = ws.numel()
+            ops.attention_prefill_mfma_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table,
+                                          ws, wo, self.scale, self.maps, blocks if blocks <= 2 * t else t)
             return
         ws, wo = ctx.work[PORTIONS_16 if n_dec else ALL_16]
         ops.attention_generic_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table,

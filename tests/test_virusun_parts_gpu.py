@@ -366,3 +366,51 @@ def test_decoding_attention_with_keys_split_over_workgroups(gpu_device, dtype, m
                                 i32([0, 1, 2, 3]), i32(lens), bt.cuda(), 3, scale, maps, splits)
         tol = 2e-5 if out_dtype == torch.float32 else 1e-2
         assert float((out.double().cpu() - want).abs().max()) < tol * float(want.abs().max())
+
+
+@pytest.mark.parametrize("maps,H,G,Dk,Dv", [(1, 4, 2, 64, 32), (2, 4, 2, 32, 64), (2, 2, 2, 64, 128), (1, 3, 1, 128, 96),
+                                            (2, 8, 4, 96, 32)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_matrix_core_attention_for_prompt_portions(gpu_device, maps, H, G, Dk, Dv, out_dtype):
+    """Three sequences (a whole prompt of 200 tokens, 70 tokens behind a cached prefix of 450 that
+    starts inside a page, 3 tokens behind 64), pages in shuffled order; the key at a page's last
+    place stands out for a few queries. One workgroup a block, and few that share the list."""
+    from pytriton_llama_amd import ops
+    from pytriton_llama_amd.engine.batch import work_items
+    torch.manual_seed(23)
+    P, pages, scale = 16, 64, 0.2
+    lens, qlens = [200, 520, 67], [200, 70, 3]
+    order = torch.randperm(pages).tolist()
+    k_pool = (torch.randn(pages, G * maps, P, Dk, dtype=torch.float64) * 5).bfloat16().double()
+    v_pool = (torch.randn(pages, G, P, Dv, dtype=torch.float64) * 5).bfloat16().double()
+    bt = torch.full((3, -(-max(lens) // P)), -1, dtype=torch.int32)
+    qs, want, at = [], [], 0
+    for r, (n, ql) in enumerate(zip(lens, qlens)):
+        k = torch.randn(n, G * maps, Dk, dtype=torch.float64)
+        v = torch.randn(n, G, Dv, dtype=torch.float64)
+        q = torch.randn(ql, H * maps, Dk, dtype=torch.float64)
+        k[P * 2 - 1] *= 2.0
+        q[-1, 0] = k[P * 2 - 1, 0] * 1.5
+        q, k, v = (t.bfloat16().double() for t in (q, k, v))
+        out = torch.zeros(ql, H * maps, Dv, dtype=torch.float64)
+        for j in range(H * maps):
+            vh = (j // maps) // (H // G)
+            s = (q[:, j] @ k[:, vh * maps + j % maps].T) * scale
+            s = s.masked_fill(torch.arange(n)[None, :] > torch.arange(n - ql, n)[:, None], float("-inf"))
+            out[:, j] = torch.softmax(s, -1) @ v[:, vh]
+        table = order[at:at + -(-n // P)]
+        at += len(table)
+        bt[r, :len(table)] = torch.tensor(table, dtype=torch.int32)
+        for i in range(n):
+            k_pool[table[i // P], :, i % P] = k[i]
+            v_pool[table[i // P], :, i % P] = v[i]
+        qs.append(q), want.append(out)
+    want = torch.cat(want)
+    ws, wo = work_items(qlens, lens, 0, 64)
+    for groups in (len(ws), 2):
+        out = torch.empty(sum(qlens), H * maps, Dv, dtype=out_dtype, device="cuda")
+        ops.attention_prefill_mfma_kv(out, dev(torch.cat(qs), torch.bfloat16), dev(k_pool, torch.bfloat16),
+                                      dev(v_pool, torch.bfloat16), i32([0, 200, 270, 273]), i32(lens), bt.cuda(),
+                                      torch.from_numpy(ws).cuda(), torch.from_numpy(wo).cuda(), scale, maps, groups)
+        # probabilities are rounded to bfloat16 for the second product
+        assert float((out.double().cpu() - want).abs().max()) < 1.5e-2 * float(want.abs().max())
