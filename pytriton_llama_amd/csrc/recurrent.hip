@@ -11,7 +11,8 @@
 // held by 16 lanes (one row of a wave for the data-parallel lane moves), each lane with R rows of it
 // in registers (D <= 16 R; rows beyond D stay zero). A step is R multiply-adds for each product
 // and a sum over the 16 lanes; the tokens of a sequence are walked in order, 16 at a time through
-// LDS, so the result does not depend on how the sequence was cut into steps. n and m of the
+// LDS (the next 16 are on their way from global memory meanwhile), so the result does not depend
+// on how the sequence was cut into steps. n and m of the
 // matrix memory are kept once per column block (every block carries the same values), so that no
 // workgroup reads what another one writes.
 //
@@ -84,48 +85,79 @@ __global__ void __launch_bounds__(256) scan_kernel(ScanArgs A) {
   }
   float m = MODE == MODE_MEMORY ? st[16 * D + D] : 0.f;
 
-  for (int t0 = 0; t0 < qlen; t0 += CHUNK) {
+  // The next 16 tokens are fetched from global memory into registers while the current 16 are
+  // worked on from LDS: a thread fetches R entries of k and of q (CHUNK * DP / 256), one of v
+  // and, the first CHUNK threads, a token's two raw gates.
+  float fk[R], fq[R], fv, fa, fb;
+  auto fetch = [&](int t0) {
     const int steps = min(CHUNK, qlen - t0);
-    __syncthreads();
-    for (int i = tid; i < CHUNK * DP; i += 256) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int i = tid + 256 * j;
       const int t = i / DP, d = i - t * DP;
-      float kv = 0.f, qv = 0.f;
+      fk[j] = 0.f;
+      fq[j] = 0.f;
       if (t < steps && d < D) {
         const size_t row = (size_t)(row0 + t0 + t);
-        kv = A.k[row * A.ldk + (size_t)g * D + d];
-        qv = A.q[row * A.ldq + (size_t)g * D + d] * A.qscale;
+        fk[j] = A.k[row * A.ldk + (size_t)g * D + d];
+        fq[j] = A.q[row * A.ldq + (size_t)g * D + d] * A.qscale;
       }
-      ks[t][d] = kv;
-      qs[t][d] = qv;
     }
-    {
-      const int t = tid >> 4, c = tid & 15;          // (256 threads: CHUNK x 16)
-      const int cc = b * 16 + c;
-      vs[t][c] = (t < steps && cc < Dv) ? A.v[(size_t)(row0 + t0 + t) * A.ldv + (size_t)h * Dv + cc] : 0.f;
-    }
+    const int cc = b * 16 + l;
+    fv = (cg < steps && cc < Dv) ? A.v[(size_t)(row0 + t0 + cg) * A.ldv + (size_t)h * Dv + cc] : 0.f;
+    fa = fb = 0.f;
     if (tid < steps) {
       const size_t row = (size_t)(row0 + t0 + tid);
-      const float a = A.ga[row * A.ldg + h], bb = A.gb[row * A.ldg + h];
+      fa = A.ga[row * A.ldg + h];
+      fb = A.gb[row * A.ldg + h];
+    }
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int i = tid + 256 * j;
+      const int t = i / DP, d = i - t * DP;
+      ks[t][d] = fk[j];
+      qs[t][d] = fq[j];
+    }
+    vs[cg][l] = fv;
+    if (tid < CHUNK) {
       if (MODE == MODE_DELTA) {
-        g0s[tid] = expf(-expf(A.c0[h]) * softplus_f(a + A.c1[h]));      // decay
-        g1s[tid] = 1.0f / (1.0f + expf(-bb));                            // beta
+        g0s[tid] = expf(-expf(A.c0[h]) * softplus_f(fa + A.c1[h]));      // decay
+        g1s[tid] = 1.0f / (1.0f + expf(-fb));                             // beta
       } else {
-        g0s[tid] = A.cap * tanhf((a + A.c0[h]) / A.cap);                 // log input gate
-        g1s[tid] = logsigmoid_f(A.cap * tanhf((bb + A.c1[h]) / A.cap));  // log forget gate
+        g0s[tid] = A.cap * tanhf((fa + A.c0[h]) / A.cap);                 // log input gate
+        g1s[tid] = logsigmoid_f(A.cap * tanhf((fb + A.c1[h]) / A.cap));   // log forget gate
       }
     }
-    __syncthreads();
+  };
+
+  fetch(0);
+  put();
+  __syncthreads();
+  for (int t0 = 0; t0 < qlen; t0 += CHUNK) {
+    const int steps = min(CHUNK, qlen - t0);
+    if (t0 + CHUNK < qlen) fetch(t0 + CHUNK);
+    // a step's k, q, v and gates are read from LDS one step ahead of their use
+    float kr[R], qr[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      kr[r] = ks[0][l * R + r];
+      qr[r] = qs[0][l * R + r];
+    }
+    float v = vs[0][cg], ga = g0s[0], gb = g1s[0];
     for (int t = 0; t < steps; ++t) {
-      float kr[R], qr[R];
+      const int tn = (t + 1) & (CHUNK - 1);
+      float kn[R], qn[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        kr[r] = ks[t][l * R + r];
-        qr[r] = qs[t][l * R + r];
+        kn[r] = ks[tn][l * R + r];
+        qn[r] = qs[tn][l * R + r];
       }
-      const float v = vs[t][cg];
+      const float vn = vs[tn][cg], gan = g0s[tn], gbn = g1s[tn];
       float o;
       if (MODE == MODE_DELTA) {
-        const float decay = g0s[t], beta = g1s[t];
+        const float decay = ga, beta = gb;
         float sk = 0.f;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -142,7 +174,7 @@ __global__ void __launch_bounds__(256) scan_kernel(ScanArgs A) {
         }
         o = row16_sum(sq);
       } else {
-        const float gi = g0s[t], gf = g1s[t];
+        const float gi = ga, gf = gb;
         const float m_new = fmaxf(gf + m, gi);
         const float keep = expf(gf + m - m_new), take = expf(gi - m_new);
         m = m_new;
@@ -160,13 +192,20 @@ __global__ void __launch_bounds__(256) scan_kernel(ScanArgs A) {
         o = sq / (fmaxf(fabsf(nq), expf(-m_new)) + 1e-6f);
       }
       if (l == 0) os[t][cg] = o;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        kr[r] = kn[r];
+        qr[r] = qn[r];
+      }
+      v = vn; ga = gan; gb = gbn;
     }
-    __syncthreads();
+    __syncthreads();              // everyone has read this chunk; its results are in os
     {
-      const int t = tid >> 4, c = tid & 15;
-      const int cc = b * 16 + c;
-      if (t < steps && cc < Dv) A.out[((size_t)(row0 + t0 + t) * A.H + h) * Dv + cc] = os[t][c];
+      const int cc = b * 16 + l;
+      if (cg < steps && cc < Dv) A.out[((size_t)(row0 + t0 + cg) * A.H + h) * Dv + cc] = os[cg][l];
     }
+    if (t0 + CHUNK < qlen) put();
+    __syncthreads();
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
