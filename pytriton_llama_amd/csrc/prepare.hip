@@ -25,6 +25,9 @@
 #define NORM_HEAD 1
 #define NORM_WHOLE 2
 
+// A token's work is cut into ``gridDim.y`` slices of whole heads (queries, then keys, then values),
+// so that the few tokens of a decode step still fill the chip. Every slice reads the whole row of
+// q and k when the norm is over the whole of them, else only its heads.
 template <typename TO>
 __global__ void __launch_bounds__(256)
 qkv_prepare_kernel(TO* __restrict__ q_out, const float* __restrict__ p, long ldp, int q_off, int k_off,
@@ -33,46 +36,55 @@ qkv_prepare_kernel(TO* __restrict__ q_out, const float* __restrict__ p, long ldp
                    const float* __restrict__ kw, float eps, int rot_dims,
                    const float* __restrict__ inv_freq, float mag, const int32_t* __restrict__ positions,
                    const int32_t* __restrict__ slots, TO* __restrict__ k_cache, TO* __restrict__ v_cache,
-                   int Hq, int Hk, int Hv, int Dk, int Dv, int page_size) {
+                   int Hq, int Hk, int Hv, int Dk, int Dv, int page_size, int heads_per_slice) {
   extern __shared__ float lds[];
-  const int nq = Hq * Dk, nk = k_off >= 0 ? Hk * Dk : 0;
-  float* raw = lds;                       // [nq + nk]: q then k, bias added
+  const bool own = k_off >= 0;
+  const int nq = Hq * Dk, nk = own ? Hk * Dk : 0;
+  const int heads_qk = Hq + (own ? Hk : 0);
+  float* raw = lds;                       // [nq + nk]: q then k, bias added (this slice's heads, or all)
   float* rs = raw + nq + nk;              // [Hq + Hk] (per head) or [2] (whole): 1 / rms
   __shared__ float scratch[16];
   const int t = blockIdx.x, tid = threadIdx.x;
+  // this slice: heads h_lo .. h_hi of q | k | v counted in one row
+  const int h_lo = blockIdx.y * heads_per_slice;
+  const int h_hi = min(h_lo + heads_per_slice, heads_qk + (own ? Hv : 0));
+  const int qk_lo = min(h_lo, heads_qk), qk_hi = min(h_hi, heads_qk);      // its q and k heads
   const float* row = p + (size_t)t * ldp;
-  for (int e = tid; e < nq; e += 256) raw[e] = row[q_off + e] + (qb ? qb[e] : 0.f);
-  for (int e = tid; e < nk; e += 256) raw[nq + e] = row[k_off + e] + (kb ? kb[e] : 0.f);
-  __syncthreads();
-  if (norm_mode == NORM_HEAD) {
-    const int wave = tid >> 6, lane = tid & 63;
-    const int heads = Hq + (nk ? Hk : 0);
-    for (int h = wave; h < heads; h += 4) {
-      const float* x = raw + (size_t)h * Dk;          // (k heads follow the q heads, same size)
+  if (qk_lo < qk_hi) {
+    const int e_lo = norm_mode == NORM_WHOLE ? 0 : qk_lo * Dk;
+    const int e_hi = norm_mode == NORM_WHOLE ? nq + nk : qk_hi * Dk;
+    for (int e = e_lo + tid; e < e_hi; e += 256)
+      raw[e] = e < nq ? row[q_off + e] + (qb ? qb[e] : 0.f) : row[k_off + e - nq] + (kb ? kb[e - nq] : 0.f);
+    __syncthreads();
+    if (norm_mode == NORM_HEAD) {
+      const int wave = tid >> 6, lane = tid & 63;
+      for (int h = qk_lo + wave; h < qk_hi; h += 4) {
+        const float* x = raw + (size_t)h * Dk;          // (k heads follow the q heads, same size)
+        float ss = 0.f;
+        for (int d = lane; d < Dk; d += 64) ss = fmaf(x[d], x[d], ss);
+        ss = wave_sum(ss);
+        if (lane == 0) rs[h] = 1.0f / sqrtf(ss / (float)Dk + eps);
+      }
+      __syncthreads();
+    } else if (norm_mode == NORM_WHOLE) {
       float ss = 0.f;
-      for (int d = lane; d < Dk; d += 64) ss = fmaf(x[d], x[d], ss);
-      ss = wave_sum(ss);
-      if (lane == 0) rs[h] = 1.0f / sqrtf(ss / (float)Dk + eps);
+      for (int e = tid; e < nq; e += 256) ss = fmaf(raw[e], raw[e], ss);
+      ss = block_sum(ss, scratch);
+      float sk = 0.f;
+      for (int e = tid; e < nk; e += 256) sk = fmaf(raw[nq + e], raw[nq + e], sk);
+      sk = block_sum(sk, scratch);
+      if (tid == 0) {
+        rs[0] = 1.0f / sqrtf(ss / (float)nq + eps);
+        rs[1] = nk ? 1.0f / sqrtf(sk / (float)nk + eps) : 0.f;
+      }
+      __syncthreads();
     }
-    __syncthreads();
-  } else if (norm_mode == NORM_WHOLE) {
-    float ss = 0.f;
-    for (int e = tid; e < nq; e += 256) ss = fmaf(raw[e], raw[e], ss);
-    ss = block_sum(ss, scratch);
-    float sk = 0.f;
-    for (int e = tid; e < nk; e += 256) sk = fmaf(raw[nq + e], raw[nq + e], sk);
-    sk = block_sum(sk, scratch);
-    if (tid == 0) {
-      rs[0] = 1.0f / sqrtf(ss / (float)nq + eps);
-      rs[1] = nk ? 1.0f / sqrtf(sk / (float)nk + eps) : 0.f;
-    }
-    __syncthreads();
   }
   const int half = rot_dims >> 1;
   const float pos = (float)positions[t];
   const int slot = slots ? slots[t] : -1;
   const int page = slot >= 0 ? slot / page_size : 0, in_page = slot >= 0 ? slot % page_size : 0;
-  for (int e = tid; e < nq + nk; e += 256) {
+  for (int e = qk_lo * Dk + tid; e < qk_hi * Dk; e += 256) {
     const bool is_k = e >= nq;
     const int i = is_k ? e - nq : e;                  // index inside q or inside k
     const int h = i / Dk, d = i - h * Dk;
@@ -97,8 +109,9 @@ qkv_prepare_kernel(TO* __restrict__ q_out, const float* __restrict__ p, long ldp
       k_cache[(((size_t)page * Hk + h) * page_size + in_page) * Dk + d] = from_float<TO>(val);
     }
   }
-  if (k_off >= 0 && slot >= 0) {
-    for (int e = tid; e < Hv * Dv; e += 256) {
+  if (own && slot >= 0 && h_hi > heads_qk) {
+    const int v_lo = max(h_lo, heads_qk) - heads_qk, v_hi = h_hi - heads_qk;
+    for (int e = v_lo * Dv + tid; e < v_hi * Dv; e += 256) {
       const int h = e / Dv, d = e - h * Dv;
       v_cache[(((size_t)page * Hv + h) * page_size + in_page) * Dv + d] =
           from_float<TO>(row[v_off + e] + (vb ? vb[e] : 0.f));
@@ -122,12 +135,22 @@ extern "C" int ptl_qkv_prepare(void* q_out, const float* p, long ldp, int q_off,
   const size_t floats = (size_t)Hq * Dk + (k_off >= 0 ? (size_t)Hk * Dk : 0) + Hq + (k_off >= 0 ? Hk : 0) + 2;
   const size_t lds = floats * sizeof(float);
   if (lds > 60 * 1024) return PTL_ERR_ARG;
+  // slices of whole heads: about 512 workgroups in all when the tokens are few, one a token when
+  // they are many
+  const int heads = Hq + (k_off >= 0 ? Hk + Hv : 0);
+  int slices = (512 + T_ - 1) / T_;
+  if (slices > heads) slices = heads;
+  if (slices < 1) slices = 1;
+  const int heads_per_slice = (heads + slices - 1) / slices;
+  slices = (heads + heads_per_slice - 1) / heads_per_slice;
+  dim3 grid(T_, slices);
 #define GO(TO)                                                                                        \
   {                                                                                                   \
-    qkv_prepare_kernel<TO><<<T_, 256, lds, st>>>((TO*)q_out, p, ldp, q_off, k_off, v_off, qb, kb, vb, \
-                                                 norm_mode, qw, kw, eps, rot_dims, inv_freq, mag,     \
-                                                 positions, slots, (TO*)k_cache, (TO*)v_cache, Hq, Hk, \
-                                                 Hv, Dk, Dv, page_size);                              \
+    qkv_prepare_kernel<TO><<<grid, 256, lds, st>>>((TO*)q_out, p, ldp, q_off, k_off, v_off, qb, kb,   \
+                                                   vb, norm_mode, qw, kw, eps, rot_dims, inv_freq,    \
+                                                   mag, positions, slots, (TO*)k_cache,               \
+                                                   (TO*)v_cache, Hq, Hk, Hv, Dk, Dv, page_size,       \
+                                                   heads_per_slice);                                  \
     return ptl_launch_status();                                                                       \
   }
   if (dtype == PTL_DTYPE_F32) GO(float)

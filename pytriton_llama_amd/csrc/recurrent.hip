@@ -138,23 +138,19 @@ __global__ void __launch_bounds__(256) scan_kernel(ScanArgs A) {
   for (int t0 = 0; t0 < qlen; t0 += CHUNK) {
     const int steps = min(CHUNK, qlen - t0);
     if (t0 + CHUNK < qlen) fetch(t0 + CHUNK);
-    // a step's k, q, v and gates are read from LDS one step ahead of their use
-    float kr[R], qr[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      kr[r] = ks[0][l * R + r];
-      qr[r] = qs[0][l * R + r];
-    }
-    float v = vs[0][cg], ga = g0s[0], gb = g1s[0];
-    for (int t = 0; t < steps; ++t) {
-      const int tn = (t + 1) & (CHUNK - 1);
-      float kn[R], qn[R];
+    // a step's k, q, v and gates are read from LDS one step ahead of their use, into one of two
+    // sets of registers in turn
+    auto read = [&](float (&kr)[R], float (&qr)[R], float& v, float& ga, float& gb, int t) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        kn[r] = ks[tn][l * R + r];
-        qn[r] = qs[tn][l * R + r];
+        kr[r] = ks[t][l * R + r];
+        qr[r] = qs[t][l * R + r];
       }
-      const float vn = vs[tn][cg], gan = g0s[tn], gbn = g1s[tn];
+      v = vs[t][cg];
+      ga = g0s[t];
+      gb = g1s[t];
+    };
+    auto step = [&](const float (&kr)[R], const float (&qr)[R], float v, float ga, float gb, int t) {
       float o;
       if (MODE == MODE_DELTA) {
         const float decay = ga, beta = gb;
@@ -192,12 +188,16 @@ __global__ void __launch_bounds__(256) scan_kernel(ScanArgs A) {
         o = sq / (fmaxf(fabsf(nq), expf(-m_new)) + 1e-6f);
       }
       if (l == 0) os[t][cg] = o;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        kr[r] = kn[r];
-        qr[r] = qn[r];
+    };
+    float k0[R], q0[R], k1[R], q1[R], v0, v1, a0, a1, b0, b1;
+    read(k0, q0, v0, a0, b0, 0);
+    for (int t = 0; t < steps; t += 2) {
+      read(k1, q1, v1, a1, b1, (t + 1) & (CHUNK - 1));
+      step(k0, q0, v0, a0, b0, t);
+      if (t + 1 < steps) {
+        read(k0, q0, v0, a0, b0, (t + 2) & (CHUNK - 1));
+        step(k1, q1, v1, a1, b1, t + 1);
       }
-      v = vn; ga = gan; gb = gbn;
     }
     __syncthreads();              // everyone has read this chunk; its results are in os
     {

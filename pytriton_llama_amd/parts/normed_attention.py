@@ -107,7 +107,9 @@ class NormedAttention(Part):
 
     def decode_splits(self, ctx, n_dec: int, device) -> int:
         """How many workgroups share one decoding sequence's keys: enough to fill the compute
-        units about four times over, never finer than one turn of a workgroup."""
+        units about twice over (measured on MI355X at batch 1 to 64 behind 2,048 keys: beyond that the
+        merging of a workgroup's key slots costs more than the shorter loops save), never finer
+        than one turn of a workgroup."""
         if self.force_decode_splits:
             return self.force_decode_splits
         lpk = 1
@@ -116,7 +118,7 @@ class NormedAttention(Part):
         turn = 2 * (256 // lpk)
         per_kv = self.num_heads // self.num_kv_heads
         base = max(1, n_dec * self.num_kv_heads * self.maps * (-(-per_kv // 4)))
-        want = -(-4 * ops.compute_units(device) // base)
+        want = -(-2 * ops.compute_units(device) // base)
         return max(1, min(want, -(-max(ctx.ctx_lens[:n_dec]) // turn), 64))
 
     def attend(self, a, q, cache, ctx, group) -> None:
