@@ -20,9 +20,9 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LENGTHS = {"V1": [5, 9, 33, 70, 130, 47], "V2": [3, 17, 40, 65, 31], "V3": [12, 50, 90, 20, 2],
-           "V4": [7, 30, 64, 81]}
+           "V4": [7, 30, 64, 81], "V5": [9, 140, 66, 35]}
 DTYPES = [torch.float32, torch.bfloat16]
-NAMES = ["V1", "V2", "V3", "V4"]
+NAMES = ["V1", "V2", "V3", "V4", "V5"]
 
 
 def read_folder(folder, weights_as=None):
@@ -245,7 +245,7 @@ def test_long_decoding_keeps_the_state(cases):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
-@pytest.mark.parametrize("name", ["V1", "V3"])
+@pytest.mark.parametrize("name", ["V1", "V3", "V5"])
 def test_cuttings_replayed_as_graphs(cases, name, dtype):
     """Decode steps and single portions replayed as HIP graphs (padded layouts: rows that belong
     to nobody, the padding state slot) against the plain model."""

@@ -90,8 +90,22 @@ def _v4():
     ])
 
 
+def _v5():
+    """Sizes that the matrix-core kernel for prompt portions and the split-KV decode kernel take, with
+    keys and values of different sizes either way (32 / 64 in the differential layers, 64 / 32 beside
+    the matrix memory), two heads a kv head, a key size of 64 in the recurrences."""
+    a = dict(heads=4, kv_heads=2, dim=32, vdim=64, scale=0.2, diff=0.35)
+    return model(180, 96, 1e-5, [
+        layer(parallel(rotary(4, 2, 64, 32, 0.15, 10000.0, 32, (4.0, 64, 8.0, 1.0)), memory(2, 64, 32, 12.0), 0.9, 1.1), 80),
+        layer(attention(**a), 72),
+        layer(delta(4, 2, 64, 32, 3), None),
+        layer(attention(**a, kv_from=1), 64),
+    ])
+
+
 # name -> (config, weight std, page size)
-VIRUSUN = {"V1": (_v1(), 0.12, 16), "V2": (_v2(), 0.15, 4), "V3": (_v3(), 0.12, 8), "V4": (_v4(), 0.12, 16)}
+VIRUSUN = {"V1": (_v1(), 0.12, 16), "V2": (_v2(), 0.15, 4), "V3": (_v3(), 0.12, 8), "V4": (_v4(), 0.12, 16),
+           "V5": (_v5(), 0.12, 16)}
 
 
 def virusun(name):
