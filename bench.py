@@ -242,11 +242,11 @@ def virusun_shape(width, layers, heads, kv_heads, dim, vdim, memory_heads, delta
     memory, differential attention that reads the keys and values two layers back, the gated delta
     rule; a dense feed-forward in each."""
     diff = {"heads": heads, "kv_heads": kv_heads, "dim": dim // 2, "vdim": vdim, "scale": (dim // 2) ** -0.5,
-            "diff": 0.6}
+            "diff": 0.8}
     left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
             "rot": {"base": 10000.0, "dims": dim // 2,
-                    "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
-    right = {"heads": memory_heads, "dim": dim, "vdim": vdim, "gate_cap": 15.0}
+                    "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}
+    right = {"heads": memory_heads, "dim": dim, "vdim": vdim, "gate_cap": 20.0}
     delta = {"heads": delta_heads, "kv_heads": delta_kv_heads, "dim": dim, "vdim": vdim, "conv": 4}
     out = []
     for i in range(layers):

@@ -105,7 +105,7 @@ def test_random_model_folder_round_trip(tmp_path):
     assert logits.shape == (5, cfg["vocab"]) and bool(torch.isfinite(logits).all())
 
 
-@pytest.mark.parametrize("dims,base,scaling", [(64, 10000.0, (4.0, 2048, 32.0, 1.0)), (12, 500.0, (2.0, 32, 4.0, 0.5)),
+@pytest.mark.parametrize("dims,base,scaling", [(64, 10000.0, (8.0, 4096, 16.0, 2.0)), (12, 500.0, (2.0, 32, 4.0, 0.5)),
                                                (32, 10000.0, (8.0, 128, 16.0, 2.0)), (8, 50.0, (1.5, 16, 3.0, 3.0))])
 def test_ramp_frequencies(dims, base, scaling):
     from pytriton_llama_amd.parts import ramp_inv_freq

@@ -150,7 +150,7 @@ def test_attention_with_keys_and_values_of_different_sizes(gpu_device, dtype, ma
 def test_heads_normed_and_gated(gpu_device, dtype, maps, per_head, act):
     from pytriton_llama_amd import ops
     torch.manual_seed(7)
-    T, H, Dv, lam, mult, eps = 29, 5, 72, 0.37, 0.6, 1e-5
+    T, H, Dv, lam, mult, eps = 29, 5, 72, 0.37, 0.55, 1e-5
     a = torch.randn(T, H * maps, Dv, dtype=torch.float64)
     gate = torch.randn(T, 11 + H * Dv, dtype=torch.float64)
     w = None if per_head is None else 1 + 0.2 * torch.randn(H * Dv if per_head else Dv, dtype=torch.float64)
@@ -181,7 +181,8 @@ def cut(total, sizes):
     return out
 
 
-@pytest.mark.parametrize("G,H,D,Dv,taps", [(1, 2, 16, 16, 4), (3, 3, 20, 36, 3), (2, 6, 40, 12, 2), (2, 2, 8, 50, 1)])
+@pytest.mark.parametrize("G,H,D,Dv,taps", [(1, 2, 16, 16, 4), (3, 3, 20, 36, 3), (2, 6, 40, 12, 2), (2, 2, 8, 50, 1),
+                                           (1, 1, 200, 24, 2), (1, 2, 136, 8, 3)])
 def test_delta_rule_in_portions_and_batches(gpu_device, G, H, D, Dv, taps):
     """Three sequences of unequal length that advance together in portions of changing size (down
     to one token, shorter than the convolution), in state slots used in any order; a slot is then
@@ -250,7 +251,8 @@ def test_delta_rule_in_portions_and_batches(gpu_device, G, H, D, Dv, taps):
     assert float((got[1] - want[1]).abs().max()) < 2e-5 * float(want[1].abs().max())
 
 
-@pytest.mark.parametrize("H,D,Dv,cap", [(2, 16, 16, 15.0), (3, 20, 36, 4.0), (1, 48, 40, 30.0), (5, 8, 8, 1.5)])
+@pytest.mark.parametrize("H,D,Dv,cap", [(2, 16, 16, 12.0), (3, 20, 36, 4.0), (1, 48, 40, 30.0), (5, 8, 8, 1.5),
+                                        (1, 256, 20, 8.0), (1, 176, 8, 6.0)])
 def test_matrix_memory_in_portions_and_batches(gpu_device, H, D, Dv, cap):
     from pytriton_llama_amd import ops
     torch.manual_seed(13)
