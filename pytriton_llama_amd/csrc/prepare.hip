@@ -1,7 +1,8 @@
 // What lies between a mixer's first projection and its attention, and between its attention (or
 // recurrence) and its output projection, for mixers whose queries and keys are normed:
 //
-// ptl_qkv_prepare: one workgroup a token. Reads the float32 row of the projection (q | k | v at
+// ptl_qkv_prepare: one workgroup a token, or several that share its heads when the tokens are few.
+//   Reads the float32 row of the projection (q | k | v at
 //   given columns), adds the biases, norms queries and keys (RMS norm over every head on its own
 //   with one weight for all heads, or over the whole of q and the whole of k with a weight of that
 //   size, or not at all), turns the first rot_dims entries of every head by the token's position
