@@ -262,6 +262,247 @@ extern "C" int ptl_memory_scan(float* out, const float* p, long ldp, int q_off, 
   return launch_scan<MODE_MEMORY>(A, n_seqs, st);
 }
 
+// ---- the matrix memory of a long prompt portion, segment by segment ---------------------------------
+// The memory's transition is a scalar (S <- keep S + take k v^T), so a long portion need not be
+// walked as one chain. Its rows are cut into segments of ``seg_len`` tokens:
+//   ptl_memory_gates      the scalar part alone, token by token (one wave a head and sequence):
+//                         m, and keep = e^(f + m - m'), take = e^(i - m'), e^(-m') of every token;
+//                         the final m goes to the slot
+//   local pass            every segment but the last, side by side, from a zero state: what the
+//                         segment adds (S, n) and the product of its keeps
+//   ptl_memory_combine    the state each segment starts from: start(p + 1) = keeps(p) start(p) + added(p)
+//   final pass            every segment, side by side, from its start state, with the read-outs;
+//                         the last one leaves the state in the slot
+// The same arithmetic a token as the walk in one chain, summed in another order.
+struct SegArgs {
+  float* out;                        // [T, H, Dv]
+  const float* q; const float* k; const float* v; long ldp;     // columns of the projection
+  const float* gates;                // [T, H, 4]: keep, take, e^(-m'), unused
+  float qscale;
+  float* state; long slot_stride;
+  float* work;                       // [n_seqs * P][H][blocks][16 D + D + 4]: a segment's start state
+  const int32_t* q_start; const int32_t* state_slots;
+  int H, D, Dv, P, seg_len;
+};
+
+template <int R, bool FINAL>
+__global__ void __launch_bounds__(256) memory_segment_kernel(SegArgs A) {
+  constexpr int DP = 16 * R;
+  __shared__ float ks[CHUNK][DP], qs[CHUNK][DP], vs[CHUNK][16], os[CHUNK][16], gs[CHUNK][4];
+  const int tid = threadIdx.x;
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int seq = blockIdx.z / A.P, seg = blockIdx.z - seq * A.P;
+  const int row0 = A.q_start[seq];
+  const int qlen = A.q_start[seq + 1] - row0;
+  const int nseg = (qlen + A.seg_len - 1) / A.seg_len;
+  if (qlen <= 0 || seg >= nseg || (!FINAL && seg == nseg - 1)) return;
+  const int t_begin = seg * A.seg_len, t_end = min(qlen, t_begin + A.seg_len);
+  const int D = A.D, Dv = A.Dv, H = A.H;
+  const int nb = (Dv + 15) >> 4;
+  const int block_floats = 16 * D + D + 4;
+  auto work_at = [&](int p) {
+    return A.work + (((size_t)(seq * A.P + p) * H + h) * nb + b) * block_floats;
+  };
+  const int cg = tid >> 4, l = tid & 15;
+  const int col = b * 16 + cg;
+  float S[R], n[R];
+  {
+    const float* from = work_at(seg);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int d = l * R + r;
+      S[r] = (FINAL && d < D && col < Dv) ? from[(size_t)cg * D + d] : 0.f;
+      n[r] = (FINAL && d < D) ? from[16 * D + d] : 0.f;
+    }
+  }
+  float kept = 1.f;                    // the product of the segment's keeps (local pass)
+
+  float fk[R], fq[R], fv, fg;
+  auto fetch = [&](int t0) {
+    const int steps = min(CHUNK, t_end - t0);
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int i = tid + 256 * j;
+      const int t = i / DP, d = i - t * DP;
+      fk[j] = 0.f;
+      fq[j] = 0.f;
+      if (t < steps && d < D) {
+        const size_t row = (size_t)(row0 + t0 + t);
+        fk[j] = A.k[row * A.ldp + (size_t)h * D + d];
+        if (FINAL) fq[j] = A.q[row * A.ldp + (size_t)h * D + d] * A.qscale;
+      }
+    }
+    const int cc = b * 16 + l;
+    fv = (cg < steps && cc < Dv) ? A.v[(size_t)(row0 + t0 + cg) * A.ldp + (size_t)h * Dv + cc] : 0.f;
+    fg = 0.f;
+    if (tid < 4 * steps) fg = A.gates[((size_t)(row0 + t0 + (tid >> 2)) * H + h) * 4 + (tid & 3)];
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int i = tid + 256 * j;
+      const int t = i / DP, d = i - t * DP;
+      ks[t][d] = fk[j];
+      if (FINAL) qs[t][d] = fq[j];
+    }
+    vs[cg][l] = fv;
+    if (tid < 4 * CHUNK) gs[tid >> 2][tid & 3] = fg;
+  };
+  fetch(t_begin);
+  put();
+  __syncthreads();
+  for (int t0 = t_begin; t0 < t_end; t0 += CHUNK) {
+    const int steps = min(CHUNK, t_end - t0);
+    if (t0 + CHUNK < t_end) fetch(t0 + CHUNK);
+    for (int t = 0; t < steps; ++t) {
+      float kr[R], qr[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        kr[r] = ks[t][l * R + r];
+        if (FINAL) qr[r] = qs[t][l * R + r];
+      }
+      const float keep = gs[t][0], take = gs[t][1];
+      const float tv = take * vs[t][cg];
+      if (FINAL) {
+        float sq = 0.f, nq = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] = fmaf(kr[r], tv, keep * S[r]);
+          n[r] = fmaf(kr[r], take, keep * n[r]);
+          sq = fmaf(S[r], qr[r], sq);
+          nq = fmaf(n[r], qr[r], nq);
+        }
+        sq = row16_sum(sq);
+        nq = row16_sum(nq);
+        const float o = sq / (fmaxf(fabsf(nq), gs[t][2]) + 1e-6f);
+        if (l == 0) os[t][cg] = o;
+      } else {
+        kept *= keep;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] = fmaf(kr[r], tv, keep * S[r]);
+          n[r] = fmaf(kr[r], take, keep * n[r]);
+        }
+      }
+    }
+    __syncthreads();
+    if (FINAL) {
+      const int cc = b * 16 + l;
+      if (cg < steps && cc < Dv) A.out[((size_t)(row0 + t0 + cg) * H + h) * Dv + cc] = os[cg][l];
+    }
+    if (t0 + CHUNK < t_end) put();
+    __syncthreads();
+  }
+  // local pass: what the segment adds, to where the next segment's start state will stand; final
+  // pass of the last segment: the state, to the slot
+  float* to = nullptr;
+  if (!FINAL) to = work_at(seg + 1);
+  else if (seg == nseg - 1)
+    to = A.state + (size_t)A.state_slots[seq] * A.slot_stride + ((size_t)h * nb + b) * block_floats;
+  if (to) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int d = l * R + r;
+      if (d < D && col < Dv) to[(size_t)cg * D + d] = S[r];
+      if (cg == 0 && d < D) to[16 * D + d] = n[r];
+    }
+    if (!FINAL && tid == 0) to[16 * D + D] = kept;
+  }
+}
+
+__global__ void __launch_bounds__(256) memory_combine_kernel(SegArgs A) {
+  const int b = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
+  const int row0 = A.q_start[seq];
+  const int qlen = A.q_start[seq + 1] - row0;
+  if (qlen <= 0) return;
+  const int nseg = (qlen + A.seg_len - 1) / A.seg_len;
+  const int nb = (A.Dv + 15) >> 4;
+  const int block_floats = 16 * A.D + A.D + 4;
+  const int live = 16 * A.D + A.D;                  // S^T of the block and n
+  const float* st = A.state + (size_t)A.state_slots[seq] * A.slot_stride + ((size_t)h * nb + b) * block_floats;
+  for (int i = threadIdx.x; i < live; i += 256) {
+    float cur = st[i];
+    for (int p = 0; p < nseg; ++p) {
+      float* w = A.work + (((size_t)(seq * A.P + p) * A.H + h) * nb + b) * block_floats;
+      if (p > 0) cur = fmaf(w[live], cur, w[i]);      // keeps(p - 1) start(p - 1) + added(p - 1)
+      w[i] = cur;
+    }
+  }
+}
+
+// One wave a (head, sequence): log gates of 64 tokens side by side, the running maximum token by
+// token, then the three exponentials side by side. The final m goes to every column block's copy.
+__global__ void __launch_bounds__(64)
+memory_gates_kernel(float* __restrict__ gates, const float* __restrict__ gi_raw, const float* __restrict__ gf_raw,
+                    long ldg, const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap,
+                    float* __restrict__ state, long slot_stride, const int32_t* __restrict__ q_start,
+                    const int32_t* __restrict__ state_slots, int H, int D, int Dv) {
+  const int h = blockIdx.x, seq = blockIdx.y, lane = threadIdx.x;
+  const int row0 = q_start[seq];
+  const int qlen = q_start[seq + 1] - row0;
+  if (qlen <= 0) return;
+  const int nb = (Dv + 15) >> 4;
+  const int block_floats = 16 * D + D + 4;
+  float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)h * nb * block_floats;
+  float m = st[16 * D + D];
+  for (int t0 = 0; t0 < qlen; t0 += 64) {
+    const int steps = min(64, qlen - t0);
+    float gi = 0.f, gf = 0.f;
+    if (lane < steps) {
+      const size_t row = (size_t)(row0 + t0 + lane);
+      gi = cap * tanhf((gi_raw[row * ldg + h] + i_bias[h]) / cap);
+      gf = logsigmoid_f(cap * tanhf((gf_raw[row * ldg + h] + f_bias[h]) / cap));
+    }
+    float m_before = 0.f, m_mine = 0.f;
+    for (int j = 0; j < steps; ++j) {
+      const float fj = __shfl(gf, j, 64), ij = __shfl(gi, j, 64);
+      const float m_new = fmaxf(fj + m, ij);
+      if (lane == j) { m_before = m; m_mine = m_new; }
+      m = m_new;
+    }
+    if (lane < steps) {
+      float* g = gates + ((size_t)(row0 + t0 + lane) * H + h) * 4;
+      g[0] = expf(gf + m_before - m_mine);
+      g[1] = expf(gi - m_mine);
+      g[2] = expf(-m_mine);
+      g[3] = m_mine;
+    }
+  }
+  for (int b = lane; b < nb; b += 64) st[(size_t)b * block_floats + 16 * D + D] = m;
+}
+
+// As ptl_memory_scan, for steps with long portions. gates float32 [T, H, 4] and work float32
+// [n_seqs * P, H * blocks * (16 D + D + 4)] are workspaces of the caller; P >= the segments of the
+// longest sequence of the step.
+extern "C" int ptl_memory_scan_segments(float* out, const float* p, long ldp, int q_off, int k_off, int v_off,
+                                        int i_off, int f_off, const float* i_bias, const float* f_bias,
+                                        float cap, float qscale, float* state, long slot_stride,
+                                        float* gates, float* work, int P, int seg_len,
+                                        const int32_t* q_start, const int32_t* state_slots, int n_seqs,
+                                        int H, int D, int Dv, hipStream_t st) {
+  if (n_seqs <= 0) return PTL_OK;
+  if (cap <= 0.f || P < 1 || seg_len < CHUNK || seg_len % CHUNK || D <= 0 || D > 256 || Dv <= 0 || H <= 0 ||
+      H > 65535 || (long)n_seqs * P > 65535 || !gates || !work)
+    return PTL_ERR_ARG;
+  const int nb = (Dv + 15) / 16;
+  memory_gates_kernel<<<dim3(H, n_seqs), 64, 0, st>>>(gates, p + i_off, p + f_off, ldp, i_bias, f_bias, cap,
+                                                       state, slot_stride, q_start, state_slots, H, D, Dv);
+  SegArgs A{out, p + q_off, p + k_off, p + v_off, ldp, gates, qscale, state, slot_stride, work, q_start,
+            state_slots, H, D, Dv, P, seg_len};
+  const dim3 grid(nb, H, n_seqs * P);
+  const int R = (D + 15) / 16;
+#define GO(RR)                                                          \
+  if (R <= RR) {                                                        \
+    if (P > 1) memory_segment_kernel<RR, false><<<grid, 256, 0, st>>>(A); \
+    memory_combine_kernel<<<dim3(nb, H, n_seqs), 256, 0, st>>>(A);      \
+    memory_segment_kernel<RR, true><<<grid, 256, 0, st>>>(A);           \
+    return ptl_launch_status();                                         \
+  }
+  GO(1) GO(2) GO(3) GO(4) GO(6) GO(8) GO(12) GO(16)
+#undef GO
+  return PTL_ERR_ARG;
+}
+
 // ---- the short convolutions in front of the delta rule -------------------------------------------
 __device__ __forceinline__ int seq_of_row(const int32_t* __restrict__ q_start, int n_seqs, int t) {
   // the last sequence whose first row is not beyond t (sequences without rows share their start

@@ -1472,12 +1472,20 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, p: torch.Tenso
     return out
 
 
+MEMORY_SEGMENT = 256          # tokens of a segment of a long portion (ptl_memory_scan_segments)
+MEMORY_SEGMENTS_FROM = 512    # rows of the longest sequence of a step from which segments are used
+
+
 def memory_scan(p: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: int, f_off: int,
                 i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float, qscale: float, state: torch.Tensor,
-                q_start: torch.Tensor, state_slots: torch.Tensor, H: int, D: int, Dv: int) -> torch.Tensor:
+                q_start: torch.Tensor, state_slots: torch.Tensor, H: int, D: int, Dv: int,
+                max_q_len: int = 0) -> torch.Tensor:
     """The matrix memory with exponential gates and a running maximum over the rows of every
     sequence, from and to the state slots. q, k (H heads of D), v (H of Dv) and the raw gates i, f
-    (H each) are columns of the float32 matrix p. Returns float32 [T, H, Dv]."""
+    (H each) are columns of the float32 matrix p. Returns float32 [T, H, Dv]. ``max_q_len``: the
+    rows of the step's longest sequence (or a bound); from MEMORY_SEGMENTS_FROM rows on the
+    sequences are worked on in segments side by side (the transition of this memory is a scalar, so
+    the segments' start states follow from what each adds and the product of its decays)."""
     _f32_rows(p, "memory_scan: p")
     T = p.shape[0]
     n = _check_scan(state, q_start, state_slots, H, D, Dv, "memory_scan")
@@ -1487,7 +1495,19 @@ def memory_scan(p: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: int,
     _f32_vec(i_bias, H, "memory_scan: i bias")
     _f32_vec(f_bias, H, "memory_scan: f bias")
     out = torch.empty((T, H, Dv), dtype=torch.float32, device=p.device)
-    _check(library.load("recurrent").ptl_memory_scan(
+    lib = library.load("recurrent")
+    segments = -(-int(max_q_len) // MEMORY_SEGMENT)
+    work_floats = n * segments * recurrent_state_floats(H, D, Dv)
+    if max_q_len >= MEMORY_SEGMENTS_FROM and n * segments <= 65535 and work_floats <= (1 << 27):
+        gates = torch.empty((T, H, 4), dtype=torch.float32, device=p.device)
+        work = torch.empty((work_floats,), dtype=torch.float32, device=p.device)
+        _check(lib.ptl_memory_scan_segments(
+            _ptr(out), _ptr(p), ctypes.c_long(p.stride(0)), int(q_off), int(k_off), int(v_off), int(i_off),
+            int(f_off), _ptr(i_bias), _ptr(f_bias), ctypes.c_float(cap), ctypes.c_float(qscale), _ptr(state),
+            ctypes.c_long(state.stride(0)), _ptr(gates), _ptr(work), int(segments), MEMORY_SEGMENT,
+            _ptr(q_start), _ptr(state_slots), n, H, D, Dv, _stream()), "memory_scan")
+        return out
+    _check(lib.ptl_memory_scan(
         _ptr(out), _ptr(p), ctypes.c_long(p.stride(0)), int(q_off), int(k_off), int(v_off), int(i_off),
         int(f_off), _ptr(i_bias), _ptr(f_bias), ctypes.c_float(cap), ctypes.c_float(qscale), _ptr(state),
         ctypes.c_long(state.stride(0)), _ptr(q_start), _ptr(state_slots), n, H, D, Dv, _stream()),

@@ -90,7 +90,8 @@ class MatrixMemory(_MatrixStateMixer):
         T, H, D, Dv = x.shape[0], self.num_heads, self.dim, self.vdim
         p = linear(x, self.proj, out_dtype=torch.float32, blocked=self.proj_blocked)
         o = ops.memory_scan(p, 0, self.k_off, self.v_off, self.i_off, self.f_off, self.i_bias, self.f_bias,
-                            self.cap, D ** -0.5, cache.state, ctx.q_start, ctx.state_slots, H, D, Dv)
+                            self.cap, D ** -0.5, cache.state, ctx.q_start, ctx.state_slots, H, D, Dv,
+                            ctx.max_q_len)
         out = torch.empty((T, H * Dv), dtype=x.dtype, device=x.device)
         ops.head_norm_gate(out, o, 1, 0.0, self.norm_weight, True, 1.0, p, self.g_off, ops.GATE_SIGMOID, self.eps)
         return out

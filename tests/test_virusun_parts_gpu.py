@@ -416,3 +416,63 @@ def test_matrix_core_attention_for_prompt_portions(gpu_device, maps, H, G, Dk, D
                                       torch.from_numpy(ws).cuda(), torch.from_numpy(wo).cuda(), scale, maps, groups)
         # probabilities are rounded to bfloat16 for the second product
         assert float((out.double().cpu() - want).abs().max()) < 1.5e-2 * float(want.abs().max())
+
+
+@pytest.mark.parametrize("H,D,Dv,cap", [(2, 32, 24, 10.0), (1, 72, 40, 3.0)])
+def test_matrix_memory_of_long_portions_in_segments(gpu_device, H, D, Dv, cap):
+    """Portions long enough to be worked on in segments side by side (with a last segment that is not
+    full, and a short sequence and a single token in the same step), then more tokens one by one
+    from the state the segments left; against the walk in one chain."""
+    from pytriton_llama_amd import ops
+    torch.manual_seed(29)
+    lens = [700, 30, 1, 530]
+    q_off, k_off, v_off, i_off, f_off = 0, H * D, 2 * H * D, 2 * H * D + H * Dv, 2 * H * D + H * Dv + H
+    cols = f_off + H
+    ib, fb = torch.randn(H, dtype=torch.float64), torch.randn(H, dtype=torch.float64) + 2
+    ps = []
+    for n in lens:
+        p = torch.randn(n + 5, cols, dtype=torch.float64)
+        p[:, i_off:] *= 3.0
+        ps.append(p)
+
+    def plain(p):
+        T = p.shape[0]
+        q = p[:, q_off:k_off].view(T, H, D) * D ** -0.5
+        k, v = p[:, k_off:v_off].view(T, H, D), p[:, v_off:i_off].view(T, H, Dv)
+        gi = cap * torch.tanh((p[:, i_off:f_off] + ib) / cap)
+        gf = torch.nn.functional.logsigmoid(cap * torch.tanh((p[:, f_off:f_off + H] + fb) / cap))
+        out = torch.zeros(T, H, Dv, dtype=torch.float64)
+        for h in range(H):
+            S, n, m = torch.zeros(D, Dv, dtype=torch.float64), torch.zeros(D, dtype=torch.float64), torch.zeros((), dtype=torch.float64)
+            for s in range(T):
+                m_new = torch.maximum(gf[s, h] + m, gi[s, h])
+                keep, take = torch.exp(gf[s, h] + m - m_new), torch.exp(gi[s, h] - m_new)
+                S, n, m = keep * S + take * torch.outer(k[s, h], v[s, h]), keep * n + take * k[s, h], m_new
+                out[s, h] = S.T @ q[s, h] / (torch.maximum((n @ q[s, h]).abs(), torch.exp(-m)) + 1e-6)
+        return out
+
+    want = [plain(p) for p in ps]
+    state = torch.randn(6, ops.recurrent_state_floats(H, D, Dv), device="cuda")
+    slot_of = [2, 5, 0, 3]
+    for s in slot_of:
+        state[s].zero_()
+    ib_d, fb_d = dev(ib), dev(fb)
+
+    def run(parts, longest):
+        p = dev(torch.cat([ps[i][lo:hi] for i, lo, hi in parts]))
+        starts = [0]
+        for _, lo, hi in parts:
+            starts.append(starts[-1] + hi - lo)
+        o = ops.memory_scan(p, q_off, k_off, v_off, i_off, f_off, ib_d, fb_d, cap, D ** -0.5, state, i32(starts),
+                            i32([slot_of[i] for i, _, _ in parts]), H, D, Dv, longest).double().cpu()
+        return [o[starts[j]:starts[j + 1]] for j in range(len(parts))]
+
+    assert max(lens) >= ops.MEMORY_SEGMENTS_FROM
+    got = run([(2, 0, 1), (0, 0, 700), (1, 0, 30), (3, 0, 530)], 700)
+    for g, i in zip(got, (2, 0, 1, 3)):
+        assert float((g - want[i][:lens[i]]).abs().max()) < 3e-5 * float(want[i].abs().max())
+    # five more tokens of each, one by one (the walk in one chain), from the states the segments left
+    for t in range(5):
+        got = run([(i, lens[i] + t, lens[i] + t + 1) for i in range(4)], 1)
+        for i, g in enumerate(got):
+            assert float((g[0] - want[i][lens[i] + t]).abs().max()) < 3e-5 * float(want[i].abs().max())
