@@ -265,7 +265,7 @@ extern "C" int ptl_memory_scan(float* out, const float* p, long ldp, int q_off, 
 // ---- the matrix memory of a long prompt portion, segment by segment ---------------------------------
 // The memory's transition is a scalar (S <- keep S + take k v^T), so a long portion need not be
 // walked as one chain. Its rows are cut into segments of ``seg_len`` tokens:
-//   ptl_memory_gates      the scalar part alone, token by token (one wave a head and sequence):
+//   the gates kernel      the scalar part alone, token by token (one workgroup a head and sequence):
 //                         m, and keep = e^(f + m - m'), take = e^(i - m'), e^(-m') of every token;
 //                         the final m goes to the slot
 //   local pass            every segment but the last, side by side, from a zero state: what the
@@ -430,14 +430,16 @@ __global__ void __launch_bounds__(256) memory_combine_kernel(SegArgs A) {
   }
 }
 
-// One wave a (head, sequence): log gates of 64 tokens side by side, the running maximum token by
-// token, then the three exponentials side by side. The final m goes to every column block's copy.
-__global__ void __launch_bounds__(64)
+// One workgroup a (head, sequence): the log gates of 256 tokens side by side, the running maximum
+// token by token (one wave, the gates read from LDS ahead of their use), then the three
+// exponentials side by side. The final m goes to every column block's copy.
+__global__ void __launch_bounds__(256)
 memory_gates_kernel(float* __restrict__ gates, const float* __restrict__ gi_raw, const float* __restrict__ gf_raw,
                     long ldg, const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap,
                     float* __restrict__ state, long slot_stride, const int32_t* __restrict__ q_start,
                     const int32_t* __restrict__ state_slots, int H, int D, int Dv) {
-  const int h = blockIdx.x, seq = blockIdx.y, lane = threadIdx.x;
+  __shared__ float gi_s[256], gf_s[256], before_s[256], after_s[256];
+  const int h = blockIdx.x, seq = blockIdx.y, tid = threadIdx.x;
   const int row0 = q_start[seq];
   const int qlen = q_start[seq + 1] - row0;
   if (qlen <= 0) return;
@@ -445,30 +447,50 @@ memory_gates_kernel(float* __restrict__ gates, const float* __restrict__ gi_raw,
   const int block_floats = 16 * D + D + 4;
   float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)h * nb * block_floats;
   float m = st[16 * D + D];
-  for (int t0 = 0; t0 < qlen; t0 += 64) {
-    const int steps = min(64, qlen - t0);
+  // the raw gates of the next 256 tokens are on their way while the current ones are worked on
+  float next_i = 0.f, next_f = 0.f;
+  if (tid < qlen) {
+    next_i = gi_raw[(size_t)(row0 + tid) * ldg + h];
+    next_f = gf_raw[(size_t)(row0 + tid) * ldg + h];
+  }
+  const float bi = i_bias[h], bf = f_bias[h];
+  for (int t0 = 0; t0 < qlen; t0 += 256) {
+    const int steps = min(256, qlen - t0);
+    const float raw_i = next_i, raw_f = next_f;
+    if (t0 + 256 + tid < qlen) {
+      next_i = gi_raw[(size_t)(row0 + t0 + 256 + tid) * ldg + h];
+      next_f = gf_raw[(size_t)(row0 + t0 + 256 + tid) * ldg + h];
+    }
     float gi = 0.f, gf = 0.f;
-    if (lane < steps) {
-      const size_t row = (size_t)(row0 + t0 + lane);
-      gi = cap * tanhf((gi_raw[row * ldg + h] + i_bias[h]) / cap);
-      gf = logsigmoid_f(cap * tanhf((gf_raw[row * ldg + h] + f_bias[h]) / cap));
+    if (tid < steps) {
+      gi = cap * tanhf((raw_i + bi) / cap);
+      gf = logsigmoid_f(cap * tanhf((raw_f + bf) / cap));
     }
-    float m_before = 0.f, m_mine = 0.f;
-    for (int j = 0; j < steps; ++j) {
-      const float fj = __shfl(gf, j, 64), ij = __shfl(gi, j, 64);
-      const float m_new = fmaxf(fj + m, ij);
-      if (lane == j) { m_before = m; m_mine = m_new; }
-      m = m_new;
+    gi_s[tid] = gi;
+    gf_s[tid] = gf;
+    __syncthreads();
+    if (tid < 64) {                       // (every lane the same values)
+#pragma unroll 8
+      for (int j = 0; j < steps; ++j) {
+        const float m_new = fmaxf(gf_s[j] + m, gi_s[j]);
+        before_s[j] = m;
+        after_s[j] = m_new;
+        m = m_new;
+      }
     }
-    if (lane < steps) {
-      float* g = gates + ((size_t)(row0 + t0 + lane) * H + h) * 4;
+    __syncthreads();
+    m = after_s[steps - 1];
+    if (tid < steps) {
+      const float m_before = before_s[tid], m_mine = after_s[tid];
+      float* g = gates + ((size_t)(row0 + t0 + tid) * H + h) * 4;
       g[0] = expf(gf + m_before - m_mine);
       g[1] = expf(gi - m_mine);
       g[2] = expf(-m_mine);
       g[3] = m_mine;
     }
+    __syncthreads();
   }
-  for (int b = lane; b < nb; b += 64) st[(size_t)b * block_floats + 16 * D + D] = m;
+  for (int b = tid; b < nb; b += 256) st[(size_t)b * block_floats + 16 * D + D] = m;
 }
 
 // As ptl_memory_scan, for steps with long portions. gates float32 [T, H, 4] and work float32
@@ -485,7 +507,7 @@ extern "C" int ptl_memory_scan_segments(float* out, const float* p, long ldp, in
       H > 65535 || (long)n_seqs * P > 65535 || !gates || !work)
     return PTL_ERR_ARG;
   const int nb = (Dv + 15) / 16;
-  memory_gates_kernel<<<dim3(H, n_seqs), 64, 0, st>>>(gates, p + i_off, p + f_off, ldp, i_bias, f_bias, cap,
+  memory_gates_kernel<<<dim3(H, n_seqs), 256, 0, st>>>(gates, p + i_off, p + f_off, ldp, i_bias, f_bias, cap,
                                                        state, slot_stride, q_start, state_slots, H, D, Dv);
   SegArgs A{out, p + q_off, p + k_off, p + v_off, ldp, gates, qscale, state, slot_stride, work, q_start,
             state_slots, H, D, Dv, P, seg_len};

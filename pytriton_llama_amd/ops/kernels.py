@@ -1472,8 +1472,8 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, p: torch.Tenso
     return out
 
 
-MEMORY_SEGMENT = 256          # tokens of a segment of a long portion (ptl_memory_scan_segments)
-MEMORY_SEGMENTS_FROM = 512    # rows of the longest sequence of a step from which segments are used
+MEMORY_SEGMENT = 128          # tokens of a segment of a long portion (measured: 64 to 512 tried at 512 to 4,096 rows)
+MEMORY_SEGMENTS_FROM = 256    # rows of the longest sequence of a step from which segments are used
 
 
 def memory_scan(p: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: int, f_off: int,
