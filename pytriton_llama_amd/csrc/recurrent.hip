@@ -525,6 +525,254 @@ extern "C" int ptl_memory_scan_segments(float* out, const float* p, long ldp, in
   return PTL_ERR_ARG;
 }
 
+// ---- the delta rule of a long prompt portion, segment by segment --------------------------------------
+// A step of the delta rule is S <- M S + beta k v^T with M = g (I - beta k k^T), the same M for every
+// column of S. Over a segment S_end = W S_start + L, where L is what the segment makes of a zero
+// state and W = M_last ... M_first is what it makes of the identity with the values left out: both
+// come from the same walk, W as D more columns. So, as for the matrix memory:
+//   local pass     every segment but the last, side by side: L (blocks of value columns) and W
+//                  (blocks of the D columns of the identity)
+//   combine        start(p + 1) = W(p) start(p) + L(p), segment after segment
+//   final pass     every segment from its start state, with the read-outs; the last leaves the
+//                  state in the slot
+// Work area of a (sequence, segment, head): [value blocks][16][D] (start state; L of the segment
+// before until the combine has run) then [key blocks][16][D] (W of the segment before, column c of
+// W as row c).
+struct DeltaSegArgs {
+  float* out;                        // [T, H, Dv]
+  const float* q; const float* k;    // [T, G, D] unit vectors
+  const float* v;                    // [T, H, Dv]
+  const float* ga; const float* gb; long ldg;     // raw gates a (decay), b (beta): [t * ldg + h]
+  const float* A_log; const float* dt_bias;
+  float* state; long slot_stride;
+  float* work;
+  const int32_t* q_start; const int32_t* state_slots;
+  int H, heads_per_qk, D, Dv, P, seg_len;
+};
+
+template <int R, bool FINAL>
+__global__ void __launch_bounds__(256) delta_segment_kernel(DeltaSegArgs A) {
+  constexpr int DP = 16 * R;
+  __shared__ float ks[CHUNK][DP], qs[CHUNK][DP], vs[CHUNK][16], os[CHUNK][16], g0s[CHUNK], g1s[CHUNK];
+  const int tid = threadIdx.x;
+  const int h = blockIdx.y;
+  const int seq = blockIdx.z / A.P, seg = blockIdx.z - seq * A.P;
+  const int row0 = A.q_start[seq];
+  const int qlen = A.q_start[seq + 1] - row0;
+  const int nseg = (qlen + A.seg_len - 1) / A.seg_len;
+  if (qlen <= 0 || seg >= nseg || (!FINAL && seg == nseg - 1)) return;
+  const int t_begin = seg * A.seg_len, t_end = min(qlen, t_begin + A.seg_len);
+  const int D = A.D, Dv = A.Dv, H = A.H, G = H / A.heads_per_qk;
+  const int nb = (Dv + 15) >> 4, nbk = (D + 15) >> 4;
+  const bool is_w = !FINAL && (int)blockIdx.x >= nb;          // a block of W's columns
+  const int b = is_w ? blockIdx.x - nb : blockIdx.x;
+  const int ncols = is_w ? D : Dv;
+  const size_t area = (size_t)(nb + nbk) * 16 * D;
+  auto work_at = [&](int p) {
+    return A.work + ((size_t)(seq * A.P + p) * H + h) * area + (is_w ? (size_t)nb * 16 * D : 0) +
+           (size_t)b * 16 * D;
+  };
+  const int cg = tid >> 4, l = tid & 15;
+  const int col = b * 16 + cg;
+  const int g = h / A.heads_per_qk;
+  float S[R];
+  {
+    const float* from = work_at(seg);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int d = l * R + r;
+      if (FINAL) S[r] = (d < D && col < Dv) ? from[(size_t)cg * D + d] : 0.f;
+      else S[r] = (is_w && d == col && d < D) ? 1.f : 0.f;
+    }
+  }
+  float fk[R], fq[R], fv, fa, fb;
+  auto fetch = [&](int t0) {
+    const int steps = min(CHUNK, t_end - t0);
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int i = tid + 256 * j;
+      const int t = i / DP, d = i - t * DP;
+      fk[j] = 0.f;
+      fq[j] = 0.f;
+      if (t < steps && d < D) {
+        const size_t at = ((size_t)(row0 + t0 + t) * G + g) * D + d;
+        fk[j] = A.k[at];
+        if (FINAL) fq[j] = A.q[at];
+      }
+    }
+    const int cc = b * 16 + l;
+    fv = (!is_w && cg < steps && cc < Dv) ? A.v[((size_t)(row0 + t0 + cg) * H + h) * Dv + cc] : 0.f;
+    fa = fb = 0.f;
+    if (tid < steps) {
+      const size_t row = (size_t)(row0 + t0 + tid);
+      fa = A.ga[row * A.ldg + h];
+      fb = A.gb[row * A.ldg + h];
+    }
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int i = tid + 256 * j;
+      const int t = i / DP, d = i - t * DP;
+      ks[t][d] = fk[j];
+      if (FINAL) qs[t][d] = fq[j];
+    }
+    vs[cg][l] = fv;
+    if (tid < CHUNK) {
+      g0s[tid] = expf(-expf(A.A_log[h]) * softplus_f(fa + A.dt_bias[h]));      // decay
+      g1s[tid] = 1.0f / (1.0f + expf(-fb));                                     // beta
+    }
+  };
+  fetch(t_begin);
+  put();
+  __syncthreads();
+  for (int t0 = t_begin; t0 < t_end; t0 += CHUNK) {
+    const int steps = min(CHUNK, t_end - t0);
+    if (t0 + CHUNK < t_end) fetch(t0 + CHUNK);
+    for (int t = 0; t < steps; ++t) {
+      float kr[R], qr[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        kr[r] = ks[t][l * R + r];
+        if (FINAL) qr[r] = qs[t][l * R + r];
+      }
+      const float decay = g0s[t], beta = g1s[t];
+      float sk = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        S[r] *= decay;
+        sk = fmaf(S[r], kr[r], sk);
+      }
+      sk = row16_sum(sk);
+      const float u = beta * (vs[t][cg] - sk);
+      if (FINAL) {
+        float sq = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] = fmaf(kr[r], u, S[r]);
+          sq = fmaf(S[r], qr[r], sq);
+        }
+        sq = row16_sum(sq);
+        if (l == 0) os[t][cg] = sq;
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) S[r] = fmaf(kr[r], u, S[r]);
+      }
+    }
+    __syncthreads();
+    if (FINAL) {
+      const int cc = b * 16 + l;
+      if (cg < steps && cc < Dv) A.out[((size_t)(row0 + t0 + cg) * H + h) * Dv + cc] = os[cg][l];
+    }
+    if (t0 + CHUNK < t_end) put();
+    __syncthreads();
+  }
+  float* to = nullptr;
+  if (!FINAL) to = work_at(seg + 1);
+  else if (seg == nseg - 1)
+    to = A.state + (size_t)A.state_slots[seq] * A.slot_stride + ((size_t)h * nb + b) * (16 * D + D + 4);
+  if (to) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int d = l * R + r;
+      if (d < D && col < ncols) to[(size_t)cg * D + d] = S[r];
+    }
+  }
+}
+
+// start(0) = the slot's state; start(p) = W(p - 1) start(p - 1) + L(p - 1). A workgroup takes a block
+// of 16 value columns of a head and walks the segments; a thread has one row d and CPG of the
+// columns, so an entry of W (column e of W lies as row e: W[d][e] at e D + d) is loaded once, side by
+// side with its neighbours in d, for all of them; the block's state lies in LDS as [e][16].
+template <int CPG>
+__global__ void __launch_bounds__(256) delta_combine_kernel(DeltaSegArgs A) {
+  extern __shared__ float cur[];                  // [D][16]
+  constexpr int GROUPS = 16 / CPG, DD = 256 / GROUPS;
+  const int b = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
+  const int row0 = A.q_start[seq];
+  const int qlen = A.q_start[seq + 1] - row0;
+  if (qlen <= 0) return;
+  const int nseg = (qlen + A.seg_len - 1) / A.seg_len;
+  const int D = A.D, H = A.H;
+  const int nb = (A.Dv + 15) >> 4, nbk = (D + 15) >> 4;
+  const size_t area = (size_t)(nb + nbk) * 16 * D;
+  const float* st = A.state + (size_t)A.state_slots[seq] * A.slot_stride + ((size_t)h * nb + b) * (16 * D + D + 4);
+  const int cols = min(16, A.Dv - b * 16);
+  const int d = threadIdx.x % DD, c0 = (threadIdx.x / DD) * CPG;
+  for (int i = threadIdx.x; i < 16 * D; i += 256) {
+    const int c = i / D, e = i - c * D;
+    cur[e * 16 + c] = c < cols ? st[i] : 0.f;
+  }
+  __syncthreads();
+  for (int p = 0; p < nseg; ++p) {
+    float* base = A.work + ((size_t)(seq * A.P + p) * H + h) * area;
+    float* mine = base + (size_t)b * 16 * D;
+    const float* W = base + (size_t)nb * 16 * D;
+    float acc[CPG];
+    if (d < D) {
+      if (p == 0) {
+#pragma unroll
+        for (int j = 0; j < CPG; ++j) acc[j] = cur[d * 16 + c0 + j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < CPG; ++j) acc[j] = c0 + j < cols ? mine[(size_t)(c0 + j) * D + d] : 0.f;   // L
+        // 32 entries of W on their way at a time: what binds here is how long one takes to come
+        for (int e0 = 0; e0 < D; e0 += 32) {
+          float w[32];
+#pragma unroll
+          for (int i = 0; i < 32; ++i) w[i] = e0 + i < D ? W[(size_t)(e0 + i) * D + d] : 0.f;
+#pragma unroll
+          for (int i = 0; i < 32; ++i) {
+            const int e = min(e0 + i, D - 1);
+#pragma unroll
+            for (int j = 0; j < CPG; ++j) acc[j] = fmaf(w[i], cur[e * 16 + c0 + j], acc[j]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (d < D) {
+#pragma unroll
+      for (int j = 0; j < CPG; ++j) {
+        cur[d * 16 + c0 + j] = acc[j];
+        if (c0 + j < cols) mine[(size_t)(c0 + j) * D + d] = acc[j];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// As ptl_delta_scan, for steps with long portions. work: float32 [n_seqs * P][H][(value blocks +
+// key blocks) * 16 * D], a workspace of the caller; P >= the segments of the step's longest sequence.
+extern "C" int ptl_delta_scan_segments(float* out, const float* q, const float* k, const float* v,
+                                       const float* ga, const float* gb, long ldg, const float* A_log,
+                                       const float* dt_bias, float* state, long slot_stride, float* work,
+                                       int P, int seg_len, const int32_t* q_start,
+                                       const int32_t* state_slots, int n_seqs, int H, int G, int D, int Dv,
+                                       hipStream_t st) {
+  if (n_seqs <= 0) return PTL_OK;
+  if (G <= 0 || H % G || P < 1 || seg_len < CHUNK || seg_len % CHUNK || D <= 0 || D > 256 || Dv <= 0 ||
+      H <= 0 || H > 65535 || (long)n_seqs * P > 65535 || !work)
+    return PTL_ERR_ARG;
+  const int nb = (Dv + 15) / 16, nbk = (D + 15) / 16;
+  DeltaSegArgs A{out, q, k, v, ga, gb, ldg, A_log, dt_bias, state, slot_stride, work, q_start, state_slots,
+                 H, H / G, D, Dv, P, seg_len};
+  const int R = (D + 15) / 16;
+  const size_t lds = (size_t)16 * D * sizeof(float);
+#define GO(RR)                                                                                           \
+  if (R <= RR) {                                                                                         \
+    if (P > 1) delta_segment_kernel<RR, false><<<dim3(nb + nbk, H, n_seqs * P), 256, 0, st>>>(A);        \
+    if (D <= 64) delta_combine_kernel<4><<<dim3(nb, H, n_seqs), 256, lds, st>>>(A);                      \
+    else if (D <= 128) delta_combine_kernel<8><<<dim3(nb, H, n_seqs), 256, lds, st>>>(A);                \
+    else delta_combine_kernel<16><<<dim3(nb, H, n_seqs), 256, lds, st>>>(A);                             \
+    delta_segment_kernel<RR, true><<<dim3(nb, H, n_seqs * P), 256, 0, st>>>(A);                          \
+    return ptl_launch_status();                                                                          \
+  }
+  GO(1) GO(2) GO(3) GO(4) GO(6) GO(8) GO(12) GO(16)
+#undef GO
+  return PTL_ERR_ARG;
+}
+
 // ---- the short convolutions in front of the delta rule -------------------------------------------
 __device__ __forceinline__ int seq_of_row(const int32_t* __restrict__ q_start, int n_seqs, int t) {
   // the last sequence whose first row is not beyond t (sequences without rows share their start

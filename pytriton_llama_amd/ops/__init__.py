@@ -14,4 +14,5 @@ from .kernels import (PROBE_MFMA_FLOPS_PER_ITER, ROWS_MIN, KernelError, RowScale
                       attention_generic_kv, attention_decode_kv, attention_decode_kv_fits, attention_prefill_mfma_kv,
                       attention_prefill_mfma_kv_fits, qkv_prepare, head_norm_gate, stream_add_rmsnorm_sum,
                       stream_rmsnorm, recurrent_block_floats, recurrent_state_floats, conv_prepare,
-                      conv_tail_update, delta_scan, memory_scan, MEMORY_SEGMENT, MEMORY_SEGMENTS_FROM)
+                      conv_tail_update, delta_scan, memory_scan, MEMORY_SEGMENT, MEMORY_SEGMENTS_FROM,
+                      DELTA_SEGMENTS_FROM, delta_segment)

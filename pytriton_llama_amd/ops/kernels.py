@@ -1446,12 +1446,27 @@ def conv_tail_update(p: torch.Tensor, x_off: int, C: int, taps: int, state: torc
         int(C), int(taps), _stream()), "conv_tail_update")
 
 
+# Segments of the delta rule (ptl_delta_scan_segments): 256 tokens, 512 from 2,048 rows on, used from
+# 768 rows on. Measured on MI355X, 16 heads of 128 x 128, one sequence, us (one chain / 128 / 256 /
+# 512): 512 rows 194 / 152 / 155 / 159; 1,024 rows 364 / 280 / 219 / 274; 2,048 rows 765 / 554 / 397 /
+# 360; 4,096 rows 1,471 / 1,104 / 764 / 611. The step from segment to segment (a D x D matrix times
+# the state, one after the other) is what short segments pay for.
+DELTA_SEGMENTS_FROM = 768
+
+
+def delta_segment(max_q_len: int) -> int:
+    return 512 if max_q_len >= 2048 else 256
+
+
 def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, p: torch.Tensor, a_off: int, b_off: int,
                A_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor,
-               state_slots: torch.Tensor) -> torch.Tensor:
+               state_slots: torch.Tensor, max_q_len: int = 0) -> torch.Tensor:
     """The gated delta rule over the rows of every sequence, from and to the state slots. q, k
     float32 [T, G, D], v float32 [T, H, Dv]; the raw gates a (decay) and b (beta) are columns
-    a_off + h and b_off + h of the float32 matrix p. Returns float32 [T, H, Dv]."""
+    a_off + h and b_off + h of the float32 matrix p. Returns float32 [T, H, Dv]. ``max_q_len``: the
+    rows of the step's longest sequence (or a bound); from DELTA_SEGMENTS_FROM rows on the
+    sequences are worked on in segments side by side (a segment's effect on the state is
+    S_end = W S_start + L; W comes from the same walk as L, started from the identity)."""
     T, G, D = q.shape
     H, Dv = v.shape[1], v.shape[2]
     _f32_rows(p, "delta_scan: p")
@@ -1465,7 +1480,18 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, p: torch.Tenso
     _f32_vec(dt_bias, H, "delta_scan: dt_bias")
     out = torch.empty((T, H, Dv), dtype=torch.float32, device=q.device)
     pa, pb = p[:, a_off:], p[:, b_off:]
-    _check(library.load("recurrent").ptl_delta_scan(
+    lib = library.load("recurrent")
+    seg_len = delta_segment(int(max_q_len))
+    segments = -(-int(max_q_len) // seg_len)
+    work_floats = n * segments * H * (-(-Dv // 16) + -(-D // 16)) * 16 * D
+    if max_q_len >= DELTA_SEGMENTS_FROM and n * segments <= 65535 and work_floats <= (1 << 27):
+        work = torch.empty((work_floats,), dtype=torch.float32, device=q.device)
+        _check(lib.ptl_delta_scan_segments(
+            _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pa), _ptr(pb), ctypes.c_long(p.stride(0)), _ptr(A_log),
+            _ptr(dt_bias), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(work), int(segments),
+            seg_len, _ptr(q_start), _ptr(state_slots), n, H, G, D, Dv, _stream()), "delta_scan")
+        return out
+    _check(lib.ptl_delta_scan(
         _ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(pa), _ptr(pb), ctypes.c_long(p.stride(0)), _ptr(A_log),
         _ptr(dt_bias), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(q_start), _ptr(state_slots), n,
         H, G, D, Dv, _stream()), "delta_scan")

@@ -168,7 +168,7 @@ class GatedDeltaRule(_MatrixStateMixer):
         ops.conv_tail_update(p, 0, self.channels, self.taps, cache.state, self.tail_off, ctx.q_start,
                              ctx.state_slots)
         o = ops.delta_scan(q, k, v, p, self.a_off, self.b_off, self.A_log, self.dt_bias, cache.state,
-                           ctx.q_start, ctx.state_slots)
+                           ctx.q_start, ctx.state_slots, ctx.max_q_len)
         out = torch.empty((T, H * Dv), dtype=x.dtype, device=x.device)
         ops.head_norm_gate(out, o, 1, 0.0, self.norm_weight, False, 1.0, p, self.g_off, ops.GATE_SILU, self.eps)
         return out

@@ -476,3 +476,63 @@ def test_matrix_memory_of_long_portions_in_segments(gpu_device, H, D, Dv, cap):
         got = run([(i, lens[i] + t, lens[i] + t + 1) for i in range(4)], 1)
         for i, g in enumerate(got):
             assert float((g[0] - want[i][lens[i] + t]).abs().max()) < 3e-5 * float(want[i].abs().max())
+
+
+@pytest.mark.parametrize("G,H,D,Dv,taps", [(1, 2, 32, 24, 3), (2, 2, 40, 72, 2)])
+def test_delta_rule_of_long_portions_in_segments(gpu_device, G, H, D, Dv, taps):
+    """Portions long enough to be worked on in segments side by side (a last segment that is not
+    full; a short sequence and a single token in the same step), then more tokens one by one from
+    the state the segments left; against the walk in one chain."""
+    from pytriton_llama_amd import ops
+    torch.manual_seed(31)
+    C = 2 * G * D + H * Dv
+    cols = C + 2 * H
+    lens = [900, 20, 1, 300]
+    cw = torch.randn(C, taps, dtype=torch.float64) * 0.5
+    A_log, dt_bias = torch.rand(H, dtype=torch.float64) * 2 - 3, torch.randn(H, dtype=torch.float64)
+    ps = [torch.randn(n + 4, cols, dtype=torch.float64) for n in lens]
+
+    def plain(p):
+        T = p.shape[0]
+        x = pv.silu(pv.short_conv(p[:, :C], cw))
+        q, k, v = x[:, :G * D].view(T, G, D), x[:, G * D:2 * G * D].view(T, G, D), x[:, 2 * G * D:].view(T, H, Dv)
+        q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+        k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+        beta = torch.sigmoid(p[:, C + H:])
+        decay = torch.exp(-torch.exp(A_log) * torch.nn.functional.softplus(p[:, C:C + H] + dt_bias))
+        out = torch.zeros(T, H, Dv, dtype=torch.float64)
+        for h in range(H):
+            S = torch.zeros(D, Dv, dtype=torch.float64)
+            for s in range(T):
+                S = decay[s, h] * S
+                S = S + torch.outer(k[s, h // (H // G)], beta[s, h] * (v[s, h] - S.T @ k[s, h // (H // G)]))
+                out[s, h] = S.T @ q[s, h // (H // G)]
+        return out
+
+    want = [plain(p) for p in ps]
+    tail_off = ops.recurrent_state_floats(H, D, Dv)
+    state = torch.randn(6, tail_off + (taps - 1) * C, device="cuda")
+    slot_of = [1, 4, 0, 5]
+    for s in slot_of:
+        state[s].zero_()
+    cw_d, A_d, dt_d = dev(cw), dev(A_log), dev(dt_bias)
+
+    def run(parts, longest):
+        p = dev(torch.cat([ps[i][lo:hi] for i, lo, hi in parts]))
+        starts = [0]
+        for _, lo, hi in parts:
+            starts.append(starts[-1] + hi - lo)
+        q_start, slots = i32(starts), i32([slot_of[i] for i, _, _ in parts])
+        q, k, v = ops.conv_prepare(p, 0, cw_d, state, tail_off, q_start, slots, G, H, D, Dv, D ** -0.5)
+        ops.conv_tail_update(p, 0, C, taps, state, tail_off, q_start, slots)
+        o = ops.delta_scan(q, k, v, p, C, C + H, A_d, dt_d, state, q_start, slots, longest).double().cpu()
+        return [o[starts[j]:starts[j + 1]] for j in range(len(parts))]
+
+    assert max(lens) >= ops.DELTA_SEGMENTS_FROM
+    got = run([(2, 0, 1), (0, 0, 900), (1, 0, 20), (3, 0, 300)], 900)
+    for g, i in zip(got, (2, 0, 1, 3)):
+        assert float((g - want[i][:lens[i]]).abs().max()) < 3e-5 * float(want[i].abs().max())
+    for t in range(4):
+        got = run([(i, lens[i] + t, lens[i] + t + 1) for i in range(4)], 1)
+        for i, g in enumerate(got):
+            assert float((g[0] - want[i][lens[i] + t]).abs().max()) < 3e-5 * float(want[i].abs().max())
