@@ -332,3 +332,32 @@ def test_command_line_and_trace_replay(cases, tmp_path):
             ref = want[torch.float32][e["id"]][fed[e["id"]]:fed[e["id"]] + n]
             assert float((got[row:row + n] - ref).abs().max() / ref.abs().max()) < 2e-5
             row, fed[e["id"]] = row + n, fed[e["id"]] + n
+
+
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
+def test_long_portions_take_the_recurrences_in_segments(cases, graphs):
+    """Portions of 900 and 300 tokens (the recurrent mixers walk them in segments side by side), the
+    first followed by portions that start inside a segment and by tokens one by one from the state
+    the segments left; launched kernel by kernel and replayed as graphs."""
+    from pytriton_llama_amd import ops
+    folders, page, _, _ = cases["V5"]
+    folder = folders[torch.float32]
+    seqs = random_sequences(180, [1240, 310], seed=21)
+    assert 900 >= ops.DELTA_SEGMENTS_FROM and 300 >= ops.MEMORY_SEGMENTS_FROM
+    want = plain_logits(folder, seqs)
+    steps, at = [], {"r0": 0, "r1": 0}
+    for rid, n in (("r0", 900), ("r1", 300), ("r0", 330), ("r1", 1), ("r1", 1)) + (("r0", 1),) * 10 + (("r1", 8),):
+        lo = at[rid]
+        at[rid] = hi = lo + n
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": seqs[rid][lo:hi], "want": [n - 1]}],
+                      "end": [rid] if hi == len(seqs[rid]) else []})
+    assert at == {r: len(t) for r, t in seqs.items()}
+    places = cuttings.wanted_places(steps)
+    if graphs:
+        runner = load_graph_runner(folder, torch.float32, page, 128, max_model_len=1280, max_num_seqs=2)
+    else:
+        runner = load_runner(folder, torch.float32, page, 128, max_num_seqs=2)
+    got = replay_wanted(runner, steps)
+    rows = {r: want[r][torch.as_tensor(places[r])] for r in got}
+    bad = first_wrong_row(got, rows, places, TOL[torch.float32])
+    assert bad is None, bad
