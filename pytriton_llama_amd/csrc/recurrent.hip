@@ -26,6 +26,8 @@
 //   x / sqrt(sum(x^2) + 1e-6) (q also times D^-1/2), all float32.
 // ptl_conv_tail_update: afterwards, the slot's last taps - 1 inputs.
 // ptl_delta_scan / ptl_memory_scan: the recurrences; gates from the float32 projection.
+// ptl_memory_scan_segments / ptl_delta_scan_segments: the same for steps with long portions, whose
+//   rows are cut into segments that are walked side by side (described where they stand, below).
 #include "common.h"
 #include <math.h>
 
